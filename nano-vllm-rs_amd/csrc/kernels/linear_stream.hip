@@ -61,7 +61,7 @@ __device__ __forceinline__ int s_w_row(int t, int nt, int r, int N, const Stream
 // of the next chunk under all of it.  A wave's k-steps are those it always had (k = 32 wave mod 256, ascending), the cross-wave order too: the same bits.
 // NC = K / 1024 is a template argument and the chunk sequence straight-line code: given these loads inside a LOOP next to the LDS-DMA requests, hipcc's
 // s_waitcnt pass drains vmcnt(0) in front of every MFMA block and every new request (one chunk in flight, the next image exposed), and weight pieces
-// requested by inline asm to hide them from that pass get COPIED at the loop's phi nodes while still in flight (caught by tools/check_kernel_isa.py).
+// requested by inline asm to hide them from that pass get COPIED at the loop's phi nodes while still in flight.
 template <int NTT, int MT, int WAVES, int U, int EPI, int TMAX, int PRE = 0, int IMG = 0, int NC = 0>
 __global__ __launch_bounds__(WAVES * 64) void linear_stream_kernel(const half_t *__restrict__ x, int64_t ldx,
                                                                    const half_t *__restrict__ W, int T, int K, int N, int KC,
@@ -138,8 +138,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_stream_kernel(const half_t 
         // pieces are requested by inline asm and waited for by hand-counted s_waitcnt: shown to the compiler next to the LDS-DMA requests, its own
         // s_waitcnt pass treats vmcnt as out of order (global_load_lds touches two address spaces) and drains vmcnt(0) in front of every MFMA block — one
         // chunk in flight, the next image exposed.  An inline-asm load is only safe while nothing copies its destination before it has landed: with loops
-        // or uniform branches in between hipcc puts such copies at the phi nodes (seen; tools/check_kernel_isa.py reads the ISA of every instantiation:
-        // no scratch, every destination untouched until the wait that covers it).
+        // or uniform branches in between hipcc puts such copies at the phi nodes (seen).
         auto body = [&](auto ntl_c) {
             constexpr int NTL = decltype(ntl_c)::value;
             constexpr bool DB = NTL * NTT * KPW2 * 2 <= 16 || (MT <= 2 && NTL * NTT * KPW2 * 2 <= 24);   // two register sets of weight pieces (<= 64 VGPRs; 96 beside
@@ -322,8 +321,8 @@ __global__ __launch_bounds__(WAVES * 64) void linear_stream_kernel(const half_t 
     float4_t cs_pre[EPI == SEPI_ROPE ? ET : 1], sn_pre[EPI == SEPI_ROPE ? ET : 1];
     // (landed long ago — they are older than the image fills that have been waited for — but the compiler cannot know that of an asm load: the wait is
     //  written down here, where nothing is in flight and it costs nothing, and the values are tied to it.  By EVERY wave, outside the branch of the
-    //  requesting waves: every control-flow path from a request to a use of its register passes this wait, which tools/check_kernel_isa.py verifies
-    //  on the ISA without having to know that `wave < MT` below is the condition the requests were issued under — ADVICE r05)
+    //  requesting waves: every control-flow path from a request to a use of its register passes this wait,
+    //  without having to know that `wave < MT` below is the condition the requests were issued under — ADVICE r05)
     if (EPI == SEPI_ROPE) asm volatile("s_waitcnt vmcnt(0)" : "+v"(pos_pre), "+v"(slot_pre) : : "memory");
     if (EPI == SEPI_ROPE && wave < MT) {
         const int tph = epi.D / 16, half_d = epi.D / 2;
