@@ -125,6 +125,10 @@ typedef struct nvr_config {
                                           arithmetic of the reference's own CPU path: its logits to ~1e-5.  nvr_runner_copy_weight then
                                           returns f32 values (two 16-bit words per element).  The stateless op entry points
                                           (nvr_linear, nvr_paged_attn_*, ...) take their 16-bit type from nvr_ops_set_dtype */
+    uint64_t num_state_slots;          /* models whose sequences carry state beside their K/V pages (recurrent state, convolution history:
+                                          nvr_model_spec_family == 1): how many sequences can hold state at once.  The block manager hands a
+                                          slot out with a sequence's blocks and takes it back with them; 0 = max_num_seqs for such a model
+                                          (an engine fills that in), none for the dense graph */
 } nvr_config;
 NVR_API void nvr_config_default(nvr_config *cfg);                    /* config.rs:54-71 */
 NVR_API int nvr_config_validate(const nvr_config *cfg);              /* config.rs:83-119 */
@@ -153,6 +157,23 @@ NVR_API void nvr_model_config_qwen3_0_6b(nvr_model_config *mc);
 NVR_API void nvr_model_config_qwen3_8b(nvr_model_config *mc);
 NVR_API int nvr_model_config_validate(const nvr_model_config *mc, uint64_t tp); /* :106-124 */
 
+/* Model registry: the text of a checkpoint's config.json -> the model family that runs it.  The 'architecture' entry (or the first of
+ * 'architectures') names a registered design: family 0 is the dense decoder graph described by nvr_model_config (Qwen3ForCausalLM: the
+ * Hugging Face keys of Qwen3Config, qwen3.rs:26-125), family 1 a LIST OF LAYERS (Rugudra: per layer a token mixer — attention with a distance
+ * penalty and a sink over the paged cache, or retention with a recurrent state — beside an optional clamped gated feed-forward, a short causal
+ * convolution in front of every sublayer, a range of layers that may run several times).  NULL + nvr_last_error for malformed text, a missing
+ * key (named in the message) or an unregistered architecture (NVR_ERR_UNSUPPORTED). */
+typedef struct nvr_model_spec nvr_model_spec_t;
+NVR_API size_t nvr_model_registry_size(void);
+NVR_API const char *nvr_model_registry_name(size_t i);
+NVR_API nvr_model_spec_t *nvr_model_spec_from_json(const char *config_json_text);
+NVR_API void nvr_model_spec_destroy(nvr_model_spec_t *spec);
+NVR_API const char *nvr_model_spec_architecture(const nvr_model_spec_t *spec);
+NVR_API int32_t nvr_model_spec_family(const nvr_model_spec_t *spec);
+NVR_API int nvr_model_spec_dense(const nvr_model_spec_t *spec, nvr_model_config *out);   /* family 0 only */
+NVR_API uint64_t nvr_model_spec_vocab(const nvr_model_spec_t *spec);
+NVR_API uint64_t nvr_model_spec_num_layer_runs(const nvr_model_spec_t *spec);           /* layers as they run (loops unrolled) */
+
 /* ------------------------------------------------------------------ Sequence ---- */
 /* Sequence, src/engine/sequence.rs:50-237.  status values = SequenceStatus :15-27 */
 typedef struct nvr_seq nvr_seq_t;
@@ -180,6 +201,11 @@ NVR_API void nvr_seq_append_token(nvr_seq_t *s, int64_t token);       /* :150 */
 NVR_API int nvr_seq_should_stop(const nvr_seq_t *s, int has_eos, int64_t eos); /* :189 */
 NVR_API void nvr_seq_preempt(nvr_seq_t *s);                           /* :213 */
 NVR_API void nvr_seq_finish(nvr_seq_t *s);                            /* :208 */
+/* A prompt that arrives in portions: n more tokens (Sequence::append_token :150 for each); and the token range the sequence contributes to the
+ * next model step that a caller builds itself (the scheduler stamps it for the steps it builds) */
+NVR_API void nvr_seq_extend(nvr_seq_t *s, const int64_t *tokens, size_t n);
+NVR_API int nvr_seq_set_chunk(nvr_seq_t *s, size_t start, size_t len);
+NVR_API int32_t nvr_seq_state_slot(const nvr_seq_t *s);              /* -1: none (nvr_bm_create_stateful) */
 
 /* -------------------------------------------------------------- BlockManager ---- */
 /* BlockManager, src/engine/block_manager.rs:69-361 */
@@ -193,6 +219,13 @@ typedef struct nvr_block_info {        /* Block :12-24 */
 
 NVR_API nvr_block_manager_t *nvr_bm_create(size_t num_blocks, size_t block_size);      /* :91 */
 NVR_API void nvr_bm_destroy(nvr_block_manager_t *bm);
+/* The same with state_slots slots of per-sequence state: allocate hands one out with the blocks (NVR_ERR_NO_FREE_BLOCKS when none is free),
+ * deallocate takes it back; blocks are then neither hashed nor shared (a cached prefix would skip tokens whose state is not in the pages).
+ * nvr_bm_extend: blocks for all tokens the sequence holds now (it grew by a portion of its prompt). */
+NVR_API nvr_block_manager_t *nvr_bm_create_stateful(size_t num_blocks, size_t block_size, size_t state_slots);
+NVR_API int nvr_bm_can_extend(const nvr_block_manager_t *bm, const nvr_seq_t *s);
+NVR_API int nvr_bm_extend(nvr_block_manager_t *bm, nvr_seq_t *s);
+NVR_API size_t nvr_bm_free_state_slots(const nvr_block_manager_t *bm);
 NVR_API uint64_t nvr_bm_compute_hash(const int64_t *tokens, size_t n, int has_prefix, uint64_t prefix); /* :109 */
 NVR_API int nvr_bm_can_allocate(const nvr_block_manager_t *bm, const nvr_seq_t *s);    /* :152 -> 0/1 */
 NVR_API int nvr_bm_allocate(nvr_block_manager_t *bm, nvr_seq_t *s);                    /* :157 */
@@ -236,6 +269,15 @@ typedef struct nvr_model_runner nvr_model_runner_t;
 
 NVR_API nvr_model_runner_t *nvr_runner_create(const nvr_config *cfg, const nvr_model_config *mc); /* :67 */
 NVR_API void nvr_runner_destroy(nvr_model_runner_t *r);
+/* A runner for whatever family the configuration names (family 0: nvr_runner_create on its nvr_model_config).  Weights are zero until
+ * loaded (nvr_runner_load_tensor by the checkpoint's tensor names). */
+NVR_API nvr_model_runner_t *nvr_runner_create_spec(const nvr_config *cfg, const nvr_model_spec_t *spec);
+/* One model step over a batch the caller built: sequence i contributes the tokens of its chunk (nvr_seq_set_chunk) — whole prompts, portions
+ * of prompts and single decoded tokens side by side, from the cache and state earlier steps left.  want_rows: rows of the step (0 .. tokens-1 in
+ * batch order) whose logits are produced, in that order (nvr_runner_copy_logits then holds n_want rows); NULL: the last row of every sequence.
+ * Family 1 models only (NVR_ERR_UNSUPPORTED otherwise: the dense graph's steps are prefill OR decode, nvr_runner_execute_model). */
+NVR_API int nvr_runner_execute_step(nvr_model_runner_t *r, nvr_seq_t *const *seqs, size_t n, const int32_t *want_rows, size_t n_want,
+                                    const float **logits_dev);
 /* :105 — logits_dev: borrowed device pointer to f32 [n, vocab/tp], valid until the next execute */
 NVR_API int nvr_runner_execute_model(nvr_model_runner_t *r, nvr_seq_t *const *seqs, size_t n, int is_prefill,
                                      const float **logits_dev);
@@ -340,6 +382,7 @@ typedef struct nvr_step_info {
 
 NVR_API nvr_engine_t *nvr_engine_create(const nvr_config *cfg, const nvr_model_config *mc); /* :34-63 */
 NVR_API void nvr_engine_destroy(nvr_engine_t *e);
+NVR_API nvr_engine_t *nvr_engine_create_spec(const nvr_config *cfg, const nvr_model_spec_t *spec);   /* any registered family */
 NVR_API int nvr_engine_add_request(nvr_engine_t *e, const int64_t *prompt, size_t n,
                                    const nvr_sampling_params *sp, uint64_t *seq_id_out);   /* :200-217 */
 NVR_API int nvr_engine_step(nvr_engine_t *e, nvr_step_info *info);                         /* :155 */

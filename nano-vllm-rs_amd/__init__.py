@@ -55,7 +55,7 @@ class ConfigC(C.Structure):
                 ("tensor_parallel_rank", C.c_uint64), ("device_ordinal", C.c_int32), ("sample_seed", C.c_uint64),
                 ("skip_block_size_check", C.c_int32), ("decode_chain", C.c_uint32),
                 ("recompute_cached_prefix", C.c_int32), ("enable_chunked_prefill", C.c_int32), ("async_decode", C.c_int32), ("shared_prefix_min_seqs", C.c_int32),
-                ("device", C.c_char * 16), ("dtype", C.c_char * 16)]
+                ("device", C.c_char * 16), ("dtype", C.c_char * 16), ("num_state_slots", C.c_uint64)]
 
 
 class ModelConfigC(C.Structure):
@@ -138,6 +138,15 @@ _SIGS = {
     "nvr_seq_block_table": (None, [_P, C.POINTER(_P), C.POINTER(C.c_size_t)]),
     "nvr_seq_append_token": (None, [_P, C.c_int64]), "nvr_seq_should_stop": (C.c_int, [_P, C.c_int, C.c_int64]),
     "nvr_seq_preempt": (None, [_P]), "nvr_seq_finish": (None, [_P]),
+    "nvr_seq_extend": (None, [_P, _P, C.c_size_t]), "nvr_seq_set_chunk": (C.c_int, [_P, C.c_size_t, C.c_size_t]), "nvr_seq_state_slot": (C.c_int32, [_P]),
+    "nvr_bm_create_stateful": (_P, [C.c_size_t, C.c_size_t, C.c_size_t]), "nvr_bm_can_extend": (C.c_int, [_P, _P]), "nvr_bm_extend": (C.c_int, [_P, _P]),
+    "nvr_bm_free_state_slots": (C.c_size_t, [_P]),
+    "nvr_model_registry_size": (C.c_size_t, []), "nvr_model_registry_name": (C.c_char_p, [C.c_size_t]),
+    "nvr_model_spec_from_json": (_P, [C.c_char_p]), "nvr_model_spec_destroy": (None, [_P]), "nvr_model_spec_architecture": (C.c_char_p, [_P]),
+    "nvr_model_spec_family": (C.c_int32, [_P]), "nvr_model_spec_dense": (C.c_int, [_P, C.POINTER(ModelConfigC)]), "nvr_model_spec_vocab": (C.c_uint64, [_P]),
+    "nvr_model_spec_num_layer_runs": (C.c_uint64, [_P]),
+    "nvr_runner_create_spec": (_P, [C.POINTER(ConfigC), _P]), "nvr_engine_create_spec": (_P, [C.POINTER(ConfigC), _P]),
+    "nvr_runner_execute_step": (C.c_int, [_P, _P, C.c_size_t, _P, C.c_size_t, C.POINTER(_P)]),
     "nvr_bm_create": (_P, [C.c_size_t, C.c_size_t]), "nvr_bm_destroy": (None, [_P]),
     "nvr_bm_compute_hash": (C.c_uint64, [_P, C.c_size_t, C.c_int, C.c_uint64]),
     "nvr_bm_can_allocate": (C.c_int, [_P, _P]), "nvr_bm_allocate": (C.c_int, [_P, _P]),
@@ -346,6 +355,55 @@ class ModelConfig:
         return self.c.head_dim or self.c.hidden_size // self.c.num_attention_heads
 
 
+class ModelSpec:
+    """A checkpoint's config.json as the model registry reads it (nvr_model_spec_from_json): which family runs the architecture it names —
+    0 the dense Qwen3 graph (ModelConfig), 1 a list of layers (Rugudra) — and that family's description.  `ModelSpec.from_pretrained(dir)` reads
+    dir/config.json; `ModelSpec(dict_or_text)` takes the configuration itself."""
+
+    def __init__(self, config):
+        import json
+        text = config if isinstance(config, str) else json.dumps(config)
+        self.h = lib().nvr_model_spec_from_json(text.encode())
+        if not self.h:
+            raise NvrError(lib().nvr_last_status() or -7, last_error())
+        self.config = json.loads(text)
+
+    @classmethod
+    def from_pretrained(cls, path: str) -> "ModelSpec":
+        with open(os.path.join(path, "config.json")) as f:
+            return cls(f.read())
+
+    def __del__(self):
+        if getattr(self, "h", None) and _lib is not None:
+            _lib.nvr_model_spec_destroy(self.h)
+            self.h = None
+
+    @property
+    def architecture(self) -> str:
+        return lib().nvr_model_spec_architecture(self.h).decode()
+
+    @property
+    def family(self) -> int:
+        return lib().nvr_model_spec_family(self.h)
+
+    @property
+    def vocab_size(self) -> int:
+        return lib().nvr_model_spec_vocab(self.h)
+
+    @property
+    def num_layer_runs(self) -> int:
+        return lib().nvr_model_spec_num_layer_runs(self.h)
+
+    def dense(self) -> "ModelConfig":
+        m = ModelConfig()
+        check(lib().nvr_model_spec_dense(self.h, C.byref(m.c)))
+        return m
+
+
+def registered_architectures() -> List[str]:
+    return [lib().nvr_model_registry_name(i).decode() for i in range(lib().nvr_model_registry_size())]
+
+
 def _read_array(fn, handle, dtype):
     p, n = _P(), C.c_size_t()
     fn(handle, C.byref(p), C.byref(n))
@@ -406,6 +464,17 @@ class Sequence:
     def last_block_num_tokens(self) -> int:
         return lib().nvr_seq_last_block_num_tokens(self.h)
 
+    def extend(self, tokens: Seq[int]) -> None:
+        a = np.ascontiguousarray(tokens, dtype=np.int64)
+        lib().nvr_seq_extend(self.h, a.ctypes.data, a.size)
+
+    def set_chunk(self, start: int, length: int) -> None:
+        check(lib().nvr_seq_set_chunk(self.h, start, length))
+
+    @property
+    def state_slot(self) -> int:
+        return lib().nvr_seq_state_slot(self.h)
+
     def append_token(self, t: int) -> None:
         lib().nvr_seq_append_token(self.h, t)
 
@@ -419,11 +488,11 @@ WAITING, RUNNING, FINISHED, PREEMPTED, ERROR = range(5)
 class BlockManager:
     """BlockManager, reference src/engine/block_manager.rs:69-361."""
 
-    def __init__(self, num_blocks: int, block_size: int, _handle=None):
+    def __init__(self, num_blocks: int, block_size: int, _handle=None, state_slots: int = 0):
         if _handle is not None:
             self.h, self.owned = _handle, False
             return
-        self.h = lib().nvr_bm_create(num_blocks, block_size)
+        self.h = lib().nvr_bm_create_stateful(num_blocks, block_size, state_slots) if state_slots else lib().nvr_bm_create(num_blocks, block_size)
         if not self.h:
             raise NvrError(-6, last_error())
         self.owned = True
@@ -446,6 +515,15 @@ class BlockManager:
 
     def deallocate(self, s: Sequence) -> None:
         check(lib().nvr_bm_deallocate(self.h, s.h))
+
+    def can_extend(self, s: Sequence) -> bool:
+        return bool(lib().nvr_bm_can_extend(self.h, s.h))
+
+    def extend(self, s: Sequence) -> None:
+        check(lib().nvr_bm_extend(self.h, s.h))
+
+    def free_state_slots(self) -> int:
+        return lib().nvr_bm_free_state_slots(self.h)
 
     def can_append(self, s: Sequence) -> bool:
         return bool(lib().nvr_bm_can_append(self.h, s.h))
@@ -573,13 +651,17 @@ class ModelRunner:
     """ModelRunner, reference src/engine/model_runner.rs:19-464."""
 
     def __init__(self, config: Config, model_config: ModelConfig, _handle=None):
-        self.vocab_local = model_config.c.vocab_size // max(1, config.c.tensor_parallel_size) if _handle is None else 0
+        self.vocab_local = model_config.c.vocab_size // max(1, config.c.tensor_parallel_size) if (_handle is None and not isinstance(model_config, ModelSpec)) else 0
         self.bf16 = bytes(config.c.dtype).split(b"\0")[0] == b"bfloat16"    # the runner's 16-bit type (Config.dtype, config.rs:51)
         self.f32 = bytes(config.c.dtype).split(b"\0")[0] == b"float32"      # the reference-precision path: 4-byte storage
         if _handle is not None:
             self.h, self.owned = _handle, False
             return
-        self.h = lib().nvr_runner_create(C.byref(config.c), C.byref(model_config.c))
+        if isinstance(model_config, ModelSpec):
+            self.vocab_local = model_config.vocab_size
+            self.h = lib().nvr_runner_create_spec(C.byref(config.c), model_config.h)
+        else:
+            self.h = lib().nvr_runner_create(C.byref(config.c), C.byref(model_config.c))
         if not self.h:
             raise NvrError(lib().nvr_last_status() or -8, last_error())
         self.owned = True
@@ -593,6 +675,18 @@ class ModelRunner:
         hs = (_P * len(seqs))(*[s.h for s in seqs])
         p = _P()
         check(lib().nvr_runner_execute_model(self.h, hs, len(seqs), int(is_prefill), C.byref(p)))
+        return p.value
+
+    def execute_step(self, seqs: List[Sequence], want_rows: Optional[Seq[int]] = None) -> int:
+        """One step over a batch the caller built (layer-list models): every sequence contributes its chunk (Sequence.set_chunk); want_rows: rows of
+        the step whose logits are produced (None: the last row of every sequence).  logits(len(want_rows)) reads them."""
+        hs = (_P * len(seqs))(*[s.h for s in seqs])
+        p = _P()
+        if want_rows is None:
+            check(lib().nvr_runner_execute_step(self.h, hs, len(seqs), None, 0, C.byref(p)))
+        else:
+            w = np.ascontiguousarray(want_rows, dtype=np.int32)
+            check(lib().nvr_runner_execute_step(self.h, hs, len(seqs), w.ctypes.data if w.size else (C.c_int32 * 1)(), w.size, C.byref(p)))
         return p.value
 
     def sample_tokens(self, seqs: List[Sequence]) -> List[int]:
@@ -815,15 +909,28 @@ def _text_args(prompts):
 class LLMEngine:
     """The hot loop of LLMEngine (reference src/engine/llm_engine.rs:155-197) over one ModelRunner."""
 
-    def __init__(self, config: Config, model_config: ModelConfig):
+    def __init__(self, config: Config, model_config):
+        """model_config: a ModelConfig (the dense graph) or a ModelSpec (whatever family the registry maps its architecture to)."""
         config.validate()
-        self.h = lib().nvr_engine_create(C.byref(config.c), C.byref(model_config.c))
+        spec = isinstance(model_config, ModelSpec)
+        self.h = lib().nvr_engine_create_spec(C.byref(config.c), model_config.h) if spec else lib().nvr_engine_create(C.byref(config.c), C.byref(model_config.c))
         if not self.h:
             raise NvrError(lib().nvr_last_status() or -8, last_error())
         self.config, self.model_config = config, model_config
         self.scheduler = Scheduler(config, _handle=lib().nvr_engine_scheduler(self.h))
         self.model_runner = ModelRunner(config, model_config, _handle=lib().nvr_engine_runner(self.h))
-        self.model_runner.vocab_local = model_config.c.vocab_size // max(1, config.c.tensor_parallel_size)
+        self.model_runner.vocab_local = model_config.vocab_size if spec else model_config.c.vocab_size // max(1, config.c.tensor_parallel_size)
+
+    @classmethod
+    def from_pretrained(cls, path: str, config: Optional[Config] = None, **kw) -> "LLMEngine":
+        """An engine for the checkpoint folder `path` (config.json + *.safetensors): the model registry picks the family by the configuration's
+        architecture, the weights are loaded by their tensor names.  kw: Config fields."""
+        spec = ModelSpec.from_pretrained(path)
+        cfg = config or Config(**kw)
+        e = cls(cfg, spec if spec.family else spec.dense())
+        e.spec = spec
+        e.model_runner.load_safetensors(path, strict=bool(spec.family))
+        return e
 
     def __del__(self):
         if getattr(self, "h", None) and _lib is not None:

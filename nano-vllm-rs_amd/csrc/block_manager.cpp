@@ -7,8 +7,9 @@
 
 namespace nvr {
 
-BlockManager::BlockManager(size_t num_blocks, size_t block_size)
-    : num_blocks_(num_blocks), block_size_(block_size), blocks_(num_blocks), arena_(num_blocks * block_size) {
+BlockManager::BlockManager(size_t num_blocks, size_t block_size, size_t state_slots)
+    : num_blocks_(num_blocks), block_size_(block_size), blocks_(num_blocks), arena_(num_blocks * block_size), state_slots_(state_slots) {
+    for (size_t i = state_slots; i-- > 0;) free_slots_.push_back((int32_t)i);
     for (size_t i = 0; i < num_blocks; ++i) list_push_back((int32_t)i);   // free ids 0..n, :96
     hash_to_block_.reserve(num_blocks * 2);
 }
@@ -68,7 +69,12 @@ int BlockManager::allocate_new_block(bool has_hash, uint64_t hash, const int64_t
 
 int BlockManager::allocate(nvr_seq &s) {                             // :157-219
     if (!s.block_table.empty()) return fail(NVR_ERR_ALREADY_ALLOCATED, "Sequence already has allocated blocks");
-    if (!can_allocate(s)) return fail(NVR_ERR_NO_FREE_BLOCKS, "Not enough free blocks to allocate sequence");
+    if (free_count_ < s.num_blocks()) return fail(NVR_ERR_NO_FREE_BLOCKS, "Not enough free blocks to allocate sequence");
+    if (state_slots_) {                                              // pages and a state slot, nothing hashed or shared
+        if (free_slots_.empty()) return fail(NVR_ERR_NO_FREE_BLOCKS, "No free state slot to allocate sequence");
+        s.state_slot = free_slots_.back(); free_slots_.pop_back();
+        return extend(s);
+    }
     bool has_prefix = false, cache_miss = false;
     uint64_t prefix = 0;
     const size_t nb = s.num_blocks();
@@ -113,11 +119,25 @@ int BlockManager::deallocate(nvr_seq &s) {                           // :240-252
     }
     s.num_cached_tokens = 0;
     s.block_table.clear();
+    if (state_slots_ && s.state_slot >= 0) { free_slots_.push_back(s.state_slot); s.state_slot = -1; }
+    return NVR_OK;
+}
+
+int BlockManager::extend(nvr_seq &s) {
+    const size_t nb = s.num_blocks();
+    if (!can_extend(s)) return fail(NVR_ERR_NO_FREE_BLOCKS, "Not enough free blocks to extend sequence");
+    while (s.block_table.size() < nb) {
+        int32_t id = -1;
+        int rc = allocate_new_block(false, 0, nullptr, 0, &id);
+        if (rc) return rc;
+        s.block_table.push_back(id);
+    }
     return NVR_OK;
 }
 
 int BlockManager::may_append(nvr_seq &s) {                           // :265-304
     if (s.block_table.empty()) return fail(NVR_ERR_NOT_ALLOCATED, "Sequence has no allocated blocks");
+    if (state_slots_) return extend(s);                              // (nothing is hashed for such models)
     const size_t last_idx = s.block_table.size() - 1;
     const int32_t last_id = s.block_table[last_idx];
     const size_t r = s.len() % block_size_;

@@ -18,16 +18,24 @@ namespace nvr {
 
 class BlockManager {
 public:
-    BlockManager(size_t num_blocks, size_t block_size);
+    // state_slots > 0: every allocated sequence also holds one of that many state slots (models whose sequences carry state beside their pages).
+    // Such a model cannot skip a prefix whose pages another sequence left behind — the state at the end of the prefix is not in the pages — so
+    // blocks are then neither hashed nor shared (num_cached_tokens stays 0).
+    BlockManager(size_t num_blocks, size_t block_size, size_t state_slots = 0);
 
     static uint64_t compute_hash(const int64_t *tokens, size_t n, bool has_prefix, uint64_t prefix);  // :109
-    bool can_allocate(const nvr_seq &s) const { return free_count_ >= s.num_blocks(); }             // :152
+    bool can_allocate(const nvr_seq &s) const { return free_count_ >= s.num_blocks() && (state_slots_ == 0 || !free_slots_.empty()); }   // :152
     int allocate(nvr_seq &s);                                                                         // :157
     int deallocate(nvr_seq &s);                                                                       // :240
     bool can_append(const nvr_seq &s) const {                                                         // :255
         return (s.len() % block_size_ == 1) ? free_count_ > 0 : true;
     }
     int may_append(nvr_seq &s);                                                                       // :265
+    // blocks for every token the sequence holds now (a prompt that arrives in portions grows by more than one token at a time)
+    bool can_extend(const nvr_seq &s) const { return s.num_blocks() <= s.block_table.size() || free_count_ >= s.num_blocks() - s.block_table.size(); }
+    int extend(nvr_seq &s);
+    size_t state_slots() const { return state_slots_; }
+    size_t free_state_slots() const { return free_slots_.size(); }
     void get_stats(nvr_bm_stats *out) const;                                                          // :307
     bool get_block(size_t id, nvr_block_info *out) const;                                             // :318
     size_t block_size() const { return block_size_; }
@@ -52,6 +60,7 @@ private:
     const int64_t *tokens_of(int32_t id) const { return arena_.data() + (size_t)id * block_size_; }
 
     size_t num_blocks_, block_size_;
+    size_t state_slots_ = 0; std::vector<int32_t> free_slots_;   // (a stack: the slot freed last is handed out first)
     std::vector<Block> blocks_;
     std::vector<int64_t> arena_;
     std::unordered_map<uint64_t, int32_t> hash_to_block_;
@@ -61,4 +70,4 @@ private:
 
 }  // namespace nvr
 
-struct nvr_block_manager { nvr::BlockManager impl; nvr_block_manager(size_t n, size_t b) : impl(n, b) {} };
+struct nvr_block_manager { nvr::BlockManager impl; nvr_block_manager(size_t n, size_t b, size_t slots = 0) : impl(n, b, slots) {} };

@@ -1,0 +1,78 @@
+// layered.h — launchers of the kernels that models described as a LIST OF LAYERS use (csrc/layered_model.cpp): a residual stream kept in
+// f32, scalar-gain RMS norms with a short causal convolution in front of every sublayer, softmax attention with a logarithmic distance
+// penalty and a sink term, retention (linear attention with a fixed decay per head, f32 state), a clamped gated feed-forward.
+//
+// One build serves both operand types: `bf16` selects 16-bit (bfloat16 bits) or f32 storage of GEMM operands, K/V cache rows and
+// weights.  Norms, angles, scores, softmax weights, the recurrence and the residual sum are f32 in both.  Every mechanism's constants
+// are arguments, none is baked in.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nvr { namespace kl {
+
+// One step's batch: row t of the step belongs to sequence row_seq[t]; the rows of sequence b are cu[b] .. cu[b+1]-1 and sit at
+// positions start[b], start[b]+1, ... of that sequence.  slot[b] is its state slot, par[b] the half of the double-buffered
+// convolution history that holds its state BEFORE this step (the step writes the other half).  Device pointers.
+struct Batch {
+    const int64_t *ids;
+    const int32_t *row_seq, *cu, *start, *slot, *par, *block_tables;
+    int32_t max_blocks, block_size, T, B, max_ctx;      // max_ctx: upper bound of start[b] + rows of b (host side)
+    int32_t max_rows;                                   // longest chunk of the step
+};
+
+int prepare();                                          // LDS opt-ins (call once, outside captures)
+
+// x[t] = E[ids[t]] * scale (f32 residual stream)
+int embed_scale(const void *E, bool bf16, const int64_t *ids, int64_t T, int64_t W, float scale, float *x, hipStream_t s);
+
+// u = x / sqrt(mean(x^2) + eps); for each of up to two consumers c: h = g_c * u, out_c[t] = h_t + sum_j w_c[:, j] * h_(t - taps + 1 + j), rows before
+// position 0 are zero and rows before the chunk come from the history hist[par][slot] ([taps-1][W] f32 rows of u); the last row of every
+// chunk writes the other half.  hist: [2][slots][taps-1][W].  out2 / w2 may be null (one consumer).  taps >= 1.
+int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, float g1, const float *w1, void *out1, float g2, const float *w2, void *out2,
+               bool bf16, float *hist, int64_t slots, hipStream_t s);
+
+// rows of K ([G][D]) and V ([G][Dv]) out of the f32 projection rows (row stride ld; column offsets kcol / vcol) into the paged caches
+// [blocks][block_size][G][D] / [..][Dv] at the rows' positions
+int kv_store(const float *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
+             hipStream_t s);
+
+// Causal softmax attention through the block tables: query row t at position i sees keys j <= i of its sequence;
+// score = q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)); the denominator also holds exp(sink[h]) (no key, no value).  r1 / r2 / sink may be null (plain
+// softmax attention).  q: f32 rows (stride ldq, heads [H][D]); out rows (stride ldo elements, heads [H][Dv]) of the operand type.
+struct SinkAttnArgs {
+    const float *q; int64_t ldq;
+    const void *kc, *vc;
+    const float *r1, *r2, *sink;
+    int32_t H, G, D, Dv; float scale;
+    void *out; int64_t ldo;
+};
+int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);
+
+// Retention over the rows of a step: per head S <- decay[h] * S + k v^T, o = S^T q, with q and k rotated (first rot_dims coordinates, pairs (i, i + rot_dims/2),
+// angle = position * freq[i]) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: f32 rows (stride ld) holding
+// q at column qcol ([H][D]), k at kcol, v at vcol ([H][Dv]).  o: f32 [T][H*Dv].
+struct RetentionArgs {
+    const float *proj; int64_t ld, qcol, kcol, vcol;
+    const float *decay, *freq; int32_t rot_dims; float kscale;
+    int32_t H, D, Dv;
+    float *state; float *o;
+};
+int retention(const RetentionArgs &a, const Batch &b, hipStream_t s);
+// out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * silu(gate[t][h*Dv + c]); gate: f32 rows (stride ldg) from column gcol
+int head_norm_gate(const float *o, const float *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
+                   hipStream_t s);
+
+// g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gu: f32 rows [T][2*F] (gate columns, then up columns)
+int clamped_glu(const float *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s);
+
+// x += mult * y (f32, [n])
+int axpy(float *x, const float *y, float mult, int64_t n, hipStream_t s);
+
+// out[r] = x[rows[r]] / sqrt(mean^2 + eps) * g, in the operand type
+int norm_rows(const float *x, const int32_t *rows, int64_t R, int64_t W, float eps, float g, void *out, bool bf16, hipStream_t s);
+
+// y[T][N] (f32) = a[T][K] . w[N][K]^T for shapes the tiled GEMMs do not take (any T, K, N)
+int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y, bool bf16, hipStream_t s);
+
+}}  // namespace nvr::kl

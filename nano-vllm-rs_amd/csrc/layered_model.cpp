@@ -1,0 +1,323 @@
+// layered_model.cpp — see layered_model.h.
+#include "layered_model.h"
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include "common.h"
+#include "model_runner.h"
+#include "kernels/kernels.h"
+
+#define RC(expr) do { int _rc = (expr); if (_rc) return _rc; } while (0)
+
+namespace nvr {
+
+namespace {
+template <class T> int dmalloc(T **p, size_t bytes) {
+    NVR_HIP_CHECK(hipMalloc((void **)p, bytes ? bytes : 16));
+    return NVR_OK;
+}
+inline float bf16_to_f(uint16_t b) { uint32_t u = (uint32_t)b << 16; float f; std::memcpy(&f, &u, 4); return f; }
+inline uint16_t f_to_bf16(float f) {
+    uint32_t u; std::memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+inline float f16_to_f(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000) << 16, exp = (h >> 10) & 0x1f, man = h & 0x3ff;
+    uint32_t u;
+    if (exp == 0) {
+        if (man == 0) u = sign;
+        else { int e = -1; uint32_t m = man; do { ++e; m <<= 1; } while (!(m & 0x400)); u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 0x3ff) << 13); }
+    } else if (exp == 31) u = sign | 0x7f800000u | (man << 13);
+    else u = sign | ((exp + 112) << 23) | (man << 13);
+    float f; std::memcpy(&f, &u, 4); return f;
+}
+inline float src_at(int dtype, const void *src, size_t i) {
+    return dtype == 2 ? ((const float *)src)[i] : dtype == 1 ? bf16_to_f(((const uint16_t *)src)[i]) : f16_to_f(((const uint16_t *)src)[i]);
+}
+}  // namespace
+
+LayeredModel::~LayeredModel() {
+    for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq})
+        if (p) (void)hipFree(p);
+    for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
+    for (void *p : {embed, head, (void *)x, (void *)proj, (void *)gu, (void *)tmp, (void *)ret_o, a1, a2, cat, xsel, (void *)in_dev}) if (p) (void)hipFree(p);
+    if (in_host) (void)hipHostFree(in_host);
+}
+
+int LayeredModel::init(nvr_model_runner &r) {
+    r.env = nvr::Env::read();
+    if (r.cfg.tensor_parallel_size != 1) return fail(NVR_ERR_UNSUPPORTED, "layer-list models run on one GPU (tensor_parallel_size 1)");
+    r.bf16 = std::strcmp(r.cfg.dtype, "bfloat16") == 0; r.f32 = std::strcmp(r.cfg.dtype, "float32") == 0;
+    if (!r.bf16 && !r.f32) return fail(NVR_ERR_UNSUPPORTED, "layer-list models: dtype '%s' (bfloat16 or float32)", r.cfg.dtype);
+    bf16 = r.bf16; esz = bf16 ? 2 : 4; r.em = bf16 ? 1 : 2;
+    r.tp = 1; r.rank = 0; r.tiled_weights = false; r.lm_fused = false;
+    const int64_t W = spec.width, V = spec.vocab;
+    r.Hd = W; r.V = r.Vl = V; r.vocab_start = 0; r.L = (int64_t)spec.runs.size();
+    r.block_size = (int64_t)r.cfg.kvcache_block_size; r.max_tokens = (int64_t)r.cfg.max_num_batched_tokens; r.max_seqs = (int64_t)r.cfg.max_num_seqs;
+    r.max_pos = std::max<int64_t>((int64_t)r.cfg.max_model_len, 1);
+    r.max_blocks_per_seq = (r.max_pos + r.block_size - 1) / r.block_size + 1;
+    slots = r.cfg.num_state_slots ? (int64_t)r.cfg.num_state_slots : r.max_seqs;
+    slot_par.assign((size_t)slots, 0);
+    r.device = r.cfg.device_ordinal;
+    NVR_HIP_CHECK(hipSetDevice(r.device));
+    NVR_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
+    RC(kl::prepare());
+    if (r.f32) RC(nvr::kf::prepare());
+    else { RC(nvr::kb::linear_stream_prepare()); RC(nvr::kb::gemm_tiled_prepare()); }
+    { int v = 0; if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, r.device) == hipSuccess && v > 0) r.num_cus = v; }
+
+    // weights (zero until loaded)
+    const int64_t taps = spec.taps;
+    int64_t max_nmix = 0, max_ff = 0, max_kcat = 0, max_hv = 0;
+    lw.resize(spec.layers.size());
+    for (size_t i = 0; i < spec.layers.size(); ++i) {
+        const LayeredSpec::Layer &L = spec.layers[i]; LayerW &w = lw[i];
+        const int64_t qn = L.heads * L.dim, kn = L.kv_heads * L.dim, vn = L.kv_heads * L.vdim, hv = L.heads * L.vdim;
+        w.qcol = 0; w.kcol = qn; w.vcol = qn + kn; w.gcol = qn + kn + vn;
+        w.nmix = qn + kn + vn + (L.mixer == LayeredSpec::RETENTION ? hv : 0);
+        w.mixcols = hv; w.kcat = hv + (L.has_mlp ? L.ff : 0);
+        RC(dmalloc(&w.mix, (size_t)(w.nmix * W * esz))); NVR_HIP_CHECK(hipMemset(w.mix, 0, (size_t)(w.nmix * W * esz)));
+        RC(dmalloc(&w.out, (size_t)(W * w.kcat * esz))); NVR_HIP_CHECK(hipMemset(w.out, 0, (size_t)(W * w.kcat * esz)));
+        if (L.has_mlp) { RC(dmalloc(&w.gu, (size_t)(2 * L.ff * W * esz))); NVR_HIP_CHECK(hipMemset(w.gu, 0, (size_t)(2 * L.ff * W * esz))); }
+        RC(dmalloc(&w.canon1, (size_t)(W * taps * 4))); NVR_HIP_CHECK(hipMemset(w.canon1, 0, (size_t)(W * taps * 4)));
+        RC(dmalloc(&w.canon2, (size_t)(W * taps * 4))); NVR_HIP_CHECK(hipMemset(w.canon2, 0, (size_t)(W * taps * 4)));
+        if (L.mixer == LayeredSpec::ATTENTION) {
+            for (float **p : {&w.r1, &w.r2, &w.sink}) { RC(dmalloc(p, (size_t)L.heads * 4)); NVR_HIP_CHECK(hipMemset(*p, 0, (size_t)L.heads * 4)); }
+        } else {
+            std::vector<float> d(L.heads), f((size_t)std::max<int64_t>(L.rot_dims / 2, 1));
+            for (int64_t h = 0; h < L.heads; ++h) d[(size_t)h] = (float)L.decay[(size_t)h];
+            for (int64_t j = 0; j < L.rot_dims / 2; ++j) f[(size_t)j] = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
+            RC(dmalloc(&w.decay, d.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.decay, d.data(), d.size() * 4, hipMemcpyHostToDevice));
+            RC(dmalloc(&w.freq, f.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.freq, f.data(), f.size() * 4, hipMemcpyHostToDevice));
+        }
+        max_nmix = std::max(max_nmix, w.nmix); max_kcat = std::max(max_kcat, w.kcat); max_hv = std::max(max_hv, hv);
+        if (L.has_mlp) max_ff = std::max(max_ff, L.ff);
+    }
+    RC(dmalloc(&embed, (size_t)(V * W * esz))); NVR_HIP_CHECK(hipMemset(embed, 0, (size_t)(V * W * esz)));
+    RC(dmalloc(&head, (size_t)(V * W * esz))); NVR_HIP_CHECK(hipMemset(head, 0, (size_t)(V * W * esz)));
+
+    // K/V pages and per-sequence state, one set per layer RUN (a looped layer keeps a cache / state per pass)
+    size_t block_bytes = 0;
+    for (int li : spec.runs) {
+        const LayeredSpec::Layer &L = spec.layers[(size_t)li];
+        if (L.mixer == LayeredSpec::ATTENTION) block_bytes += (size_t)(r.block_size * L.kv_heads * (L.dim + L.vdim) * esz);
+    }
+    if (r.cfg.num_kvcache_blocks >= 0) r.num_blocks = r.cfg.num_kvcache_blocks;
+    else if (r.cfg.num_kvcache_blocks == -1) r.num_blocks = 1000;
+    else {
+        size_t free_b = 0, total_b = 0;
+        NVR_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        const double budget = (double)free_b - (1.0 - r.cfg.gpu_memory_utilization) * (double)total_b;
+        const int64_t nb = block_bytes ? (int64_t)(budget * 0.9 / (double)block_bytes) : 1000;
+        if (nb < 1) return fail(NVR_ERR_HIP, "not enough free HBM for one KV block");
+        r.num_blocks = nb;
+    }
+    rs.resize(spec.runs.size());
+    for (size_t ri = 0; ri < spec.runs.size(); ++ri) {
+        const LayeredSpec::Layer &L = spec.layers[(size_t)spec.runs[ri]]; RunState &s = rs[ri];
+        if (L.mixer == LayeredSpec::ATTENTION) {
+            const size_t kb = (size_t)(r.num_blocks * r.block_size * L.kv_heads * L.dim * esz), vb = (size_t)(r.num_blocks * r.block_size * L.kv_heads * L.vdim * esz);
+            RC(dmalloc(&s.kc, kb)); NVR_HIP_CHECK(hipMemset(s.kc, 0, kb));
+            RC(dmalloc(&s.vc, vb)); NVR_HIP_CHECK(hipMemset(s.vc, 0, vb));
+        } else {
+            const size_t sb = (size_t)(slots * L.heads * L.dim * L.vdim * 4);
+            RC(dmalloc(&s.state, sb)); NVR_HIP_CHECK(hipMemset(s.state, 0, sb));
+        }
+        const size_t hb = (size_t)(2 * slots * (taps - 1) * W * 4);
+        RC(dmalloc(&s.hist, hb)); NVR_HIP_CHECK(hipMemset(s.hist, 0, hb ? hb : 16));
+    }
+
+    // activations
+    const int64_t MT = r.max_tokens;
+    RC(dmalloc(&x, (size_t)(MT * W * 4))); RC(dmalloc(&tmp, (size_t)(MT * W * 4)));
+    RC(dmalloc(&proj, (size_t)(MT * max_nmix * 4))); RC(dmalloc(&gu, (size_t)(MT * 2 * max_ff * 4))); RC(dmalloc(&ret_o, (size_t)(MT * max_hv * 4)));
+    RC(dmalloc(&a1, (size_t)(MT * W * esz))); RC(dmalloc(&a2, (size_t)(MT * W * esz))); RC(dmalloc(&cat, (size_t)(MT * max_kcat * esz)));
+    logit_rows_cap = std::max<int64_t>(r.max_seqs, 64);
+    RC(dmalloc(&xsel, (size_t)(std::max(MT, logit_rows_cap) * W * esz)));
+    RC(dmalloc(&r.logits, (size_t)(logit_rows_cap * V * 4)));
+
+    // step inputs: ids | row_seq | want | cu | start | slot | par | block tables
+    in_bytes = (size_t)(MT * 8 + MT * 4 * 2 + (r.max_seqs + 1) * 4 + r.max_seqs * 4 * 3 + r.max_seqs * r.max_blocks_per_seq * 4 + 256);
+    NVR_HIP_CHECK(hipHostMalloc((void **)&in_host, in_bytes, hipHostMallocDefault));
+    NVR_HIP_CHECK(hipMalloc((void **)&in_dev, in_bytes));
+
+    // sampling (Sampler::sample, sampler.rs:71-218: the runner's own samplers read r.logits)
+    NVR_HIP_CHECK(hipMalloc((void **)&r.d_tok, (size_t)r.max_seqs * 8)); NVR_HIP_CHECK(hipMalloc((void **)&r.d_maxval, (size_t)r.max_seqs * 4));
+    NVR_HIP_CHECK(hipHostMalloc((void **)&r.h_tok, (size_t)r.max_seqs * 8, hipHostMallocDefault));
+    NVR_HIP_CHECK(hipMalloc((void **)&r.d_temp, (size_t)r.max_seqs * 4)); NVR_HIP_CHECK(hipMalloc((void **)&r.d_topk, (size_t)r.max_seqs * 8));
+    NVR_HIP_CHECK(hipMalloc((void **)&r.d_topp, (size_t)r.max_seqs * 4)); NVR_HIP_CHECK(hipMalloc((void **)&r.d_keys, (size_t)r.max_seqs * 8));
+    NVR_HIP_CHECK(hipHostMalloc((void **)&r.samp_host, (size_t)r.max_seqs * 24, hipHostMallocDefault));
+    NVR_HIP_CHECK(hipMalloc(&r.sample_ws, nvr::kb::sample_workspace_bytes(r.max_seqs, V)));
+    NVR_HIP_CHECK(hipDeviceSynchronize());
+    return NVR_OK;
+}
+
+// src [rows][cols] (row-major, dtype 0 f16 / 1 bf16 / 2 f32) -> dst rows of dst_ld elements: the operand type, or f32
+int LayeredModel::put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand) {
+    const size_t n = (size_t)(rows * cols);
+    const int64_t e = (as_operand && bf16) ? 2 : 4;
+    std::vector<char> buf(n * (size_t)e);
+    if (e == 2) {
+        uint16_t *o = (uint16_t *)buf.data();
+        if (dtype == 1) std::memcpy(o, src, n * 2);
+        else for (size_t i = 0; i < n; ++i) o[i] = f_to_bf16(src_at(dtype, src, i));
+    } else {
+        float *o = (float *)buf.data();
+        for (size_t i = 0; i < n; ++i) o[i] = src_at(dtype, src, i);
+    }
+    NVR_HIP_CHECK(hipSetDevice(r.device));
+    NVR_HIP_CHECK(hipMemcpy2D(dst, (size_t)(dst_ld * e), buf.data(), (size_t)(cols * e), (size_t)(cols * e), (size_t)rows, hipMemcpyHostToDevice));
+    return NVR_OK;
+}
+
+// Tensors by the names of the checkpoint: "embed", "head", "final.norm", and per layer i "l<i>.norm1" / "norm2" (one number each), "l<i>.canon1" / "canon2"
+// [width][taps], "l<i>.mix.{q,k,v,g,o}" (+ "r1", "r2", "sink" per head for attention), "l<i>.mlp.{gate,up,down}".  Linear weights are [out][in].
+int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtype, const int64_t *shape, int ndim, const void *data) {
+    if (dtype < 0 || dtype > 2) return fail(NVR_ERR_INVALID_ARG, "load_tensor: dtype %d", dtype);
+    const std::string name(name_in);
+    const int64_t W = spec.width, V = spec.vocab;
+    auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
+    auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
+    auto scalar = [&](float *out) { int64_t n = 1; for (int i = 0; i < ndim; ++i) n *= shape[i]; if (n != 1) return bad(); *out = src_at(dtype, data, 0); return (int)NVR_OK; };
+    if (name == "embed") return is2(V, W) ? put(r, embed, W, V, W, dtype, data, true) : bad();
+    if (name == "head") return is2(V, W) ? put(r, head, W, V, W, dtype, data, true) : bad();
+    if (name == "final.norm") return scalar(&gfinal);
+    if (name.size() < 3 || name[0] != 'l') return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in);
+    size_t dot = name.find('.');
+    if (dot == std::string::npos || dot < 2) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in);
+    int64_t li = 0;
+    for (size_t i = 1; i < dot; ++i) { if (name[i] < '0' || name[i] > '9') return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in); li = li * 10 + (name[i] - '0'); }
+    if (li >= (int64_t)spec.layers.size()) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: '%s' names a layer the model does not have", name_in);
+    const LayeredSpec::Layer &L = spec.layers[(size_t)li]; LayerW &w = lw[(size_t)li];
+    const std::string rest = name.substr(dot + 1);
+    const int64_t qn = L.heads * L.dim, kn = L.kv_heads * L.dim, vn = L.kv_heads * L.vdim, hv = L.heads * L.vdim;
+    auto rows_at = [&](void *base, int64_t row0, int64_t ld) { return (void *)((char *)base + (size_t)(row0 * ld * esz)); };
+    auto vec = [&](float *dst, int64_t n) { return (ndim == 1 && shape[0] == n) ? put(r, dst, n, 1, n, dtype, data, false) : bad(); };
+    if (rest == "norm1") return scalar(&w.g1);
+    if (rest == "norm2") return scalar(&w.g2);
+    if (rest == "canon1") return is2(W, spec.taps) ? put(r, w.canon1, spec.taps, W, spec.taps, dtype, data, false) : bad();
+    if (rest == "canon2") return is2(W, spec.taps) ? put(r, w.canon2, spec.taps, W, spec.taps, dtype, data, false) : bad();
+    if (rest == "mix.q") return is2(qn, W) ? put(r, rows_at(w.mix, w.qcol, W), W, qn, W, dtype, data, true) : bad();
+    if (rest == "mix.k") return is2(kn, W) ? put(r, rows_at(w.mix, w.kcol, W), W, kn, W, dtype, data, true) : bad();
+    if (rest == "mix.v") return is2(vn, W) ? put(r, rows_at(w.mix, w.vcol, W), W, vn, W, dtype, data, true) : bad();
+    if (rest == "mix.o") return is2(W, hv) ? put(r, w.out, w.kcat, W, hv, dtype, data, true) : bad();
+    if (L.mixer == LayeredSpec::RETENTION && rest == "mix.g") return is2(hv, W) ? put(r, rows_at(w.mix, w.gcol, W), W, hv, W, dtype, data, true) : bad();
+    if (L.mixer == LayeredSpec::ATTENTION) {
+        if (rest == "mix.r1") return vec(w.r1, L.heads);
+        if (rest == "mix.r2") return vec(w.r2, L.heads);
+        if (rest == "mix.sink") return vec(w.sink, L.heads);
+    }
+    if (L.has_mlp) {
+        if (rest == "mlp.gate") return is2(L.ff, W) ? put(r, w.gu, W, L.ff, W, dtype, data, true) : bad();
+        if (rest == "mlp.up") return is2(L.ff, W) ? put(r, rows_at(w.gu, L.ff, W), W, L.ff, W, dtype, data, true) : bad();
+        if (rest == "mlp.down") return is2(W, L.ff) ? put(r, (char *)w.out + (size_t)(hv * esz), w.kcat, W, L.ff, dtype, data, true) : bad();
+    }
+    return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in);
+}
+
+int LayeredModel::gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y) {
+    if (!bf16) return nvr::kf::linear((const float *)a, lda, (const float *)w, T, K, N, nullptr, y, r.stream);
+    if (K % 32 == 0 && N % 16 == 0 && lda % 8 == 0) return nvr::kb::linear((const uint16_t *)a, lda, (const uint16_t *)w, T, K, N, y, true, r.stream);
+    return kl::gemm_any(a, lda, w, T, K, N, y, true, r.stream);
+}
+
+// One step over a batch of chunks: sequence i contributes its tokens [chunk_start, chunk_start + chunk_len).  want: rows of the step (in batch
+// order) whose logits are produced, or null for the last row of every sequence.
+int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq, const int32_t *want, size_t nwant) {
+    NVR_HIP_CHECK(hipSetDevice(r.device));
+    if (nseq == 0) return fail(NVR_ERR_INVALID_ARG, "execute_model: empty batch");
+    if ((int64_t)nseq > r.max_seqs) return fail(NVR_ERR_INVALID_ARG, "execute_model: %zu sequences exceed max_num_seqs %ld", nseq, (long)r.max_seqs);
+    int64_t T = 0, max_ctx = 0, max_rows = 0;
+    for (size_t i = 0; i < nseq; ++i) {
+        const nvr_seq *s = seqs[i];
+        if (s->chunk_len == 0 || s->chunk_start + s->chunk_len > s->num_tokens)
+            return fail(NVR_ERR_INVALID_ARG, "execute_model: sequence %lu has no valid chunk (%zu + %zu of %zu tokens)", (unsigned long)s->seq_id, s->chunk_start, s->chunk_len, s->num_tokens);
+        if (s->state_slot < 0 || s->state_slot >= slots) return fail(NVR_ERR_NOT_ALLOCATED, "execute_model: sequence %lu holds no state slot", (unsigned long)s->seq_id);
+        const int64_t end = (int64_t)(s->chunk_start + s->chunk_len);
+        if (end > r.max_pos) return fail(NVR_ERR_INVALID_ARG, "execute_model: sequence %lu reaches position %ld (max_model_len %ld)", (unsigned long)s->seq_id, (long)end, (long)r.max_pos);
+        if ((int64_t)s->block_table.size() * r.block_size < end) return fail(NVR_ERR_NOT_ALLOCATED, "execute_model: sequence %lu has blocks for %zu tokens, needs %ld", (unsigned long)s->seq_id, s->block_table.size() * (size_t)r.block_size, (long)end);
+        for (size_t j = 0; j < nseq; ++j) if (j != i && seqs[j]->state_slot == s->state_slot) return fail(NVR_ERR_INVARIANT, "execute_model: two sequences of the batch share state slot %d", s->state_slot);
+        T += (int64_t)s->chunk_len; max_ctx = std::max(max_ctx, end); max_rows = std::max<int64_t>(max_rows, (int64_t)s->chunk_len);
+    }
+    if (T > r.max_tokens) return fail(NVR_ERR_INVALID_ARG, "execute_model: %ld tokens exceed max_num_batched_tokens %ld", (long)T, (long)r.max_tokens);
+    const size_t R = want ? nwant : nseq;
+    if ((int64_t)R > std::max(r.max_tokens, logit_rows_cap)) return fail(NVR_ERR_INVALID_ARG, "execute_model: %zu rows of logits asked of a step of %ld tokens", R, (long)T);
+    if ((int64_t)R > logit_rows_cap) {                                   // (grown outside any capture: an allocation synchronises)
+        NVR_HIP_CHECK(hipStreamSynchronize(r.stream));
+        (void)hipFree(r.logits); r.logits = nullptr;
+        logit_rows_cap = (int64_t)R;
+        NVR_HIP_CHECK(hipMalloc((void **)&r.logits, (size_t)(logit_rows_cap * spec.vocab * 4)));
+    }
+    // arena
+    const int64_t MB = r.max_blocks_per_seq;
+    size_t off = 0;
+    auto carve = [&](size_t bytes) { size_t o = off; off += (bytes + 15) / 16 * 16; return o; };
+    const size_t o_ids = carve((size_t)T * 8), o_rs = carve((size_t)T * 4), o_want = carve(std::max<size_t>(R, 1) * 4), o_cu = carve((nseq + 1) * 4), o_st = carve(nseq * 4),
+                 o_sl = carve(nseq * 4), o_par = carve(nseq * 4), o_bt = carve(nseq * (size_t)MB * 4);
+    if (off > in_bytes) return fail(NVR_ERR_INVARIANT, "execute_model: step inputs of %zu bytes exceed the arena", off);
+    int64_t *ids = (int64_t *)(in_host + o_ids); int32_t *rowseq = (int32_t *)(in_host + o_rs), *wnt = (int32_t *)(in_host + o_want), *cu = (int32_t *)(in_host + o_cu),
+            *stt = (int32_t *)(in_host + o_st), *sl = (int32_t *)(in_host + o_sl), *par = (int32_t *)(in_host + o_par), *bt = (int32_t *)(in_host + o_bt);
+    int64_t t = 0;
+    for (size_t i = 0; i < nseq; ++i) {
+        const nvr_seq *s = seqs[i];
+        cu[i] = (int32_t)t; stt[i] = (int32_t)s->chunk_start; sl[i] = s->state_slot;
+        if (s->chunk_start == 0) slot_par[(size_t)s->state_slot] = 0;     // a sequence's first tokens read no history: whatever the slot held is dead
+        par[i] = slot_par[(size_t)s->state_slot];
+        for (size_t j = 0; j < s->chunk_len; ++j, ++t) {
+            const int64_t id = s->token_ids[s->chunk_start + j];
+            if ((uint64_t)id >= (uint64_t)spec.vocab) return fail(NVR_ERR_INVALID_ARG, "execute_model: token id %ld outside the vocabulary [0, %ld)", (long)id, (long)spec.vocab);
+            ids[t] = id; rowseq[t] = (int32_t)i;
+        }
+        for (int64_t j = 0; j < MB; ++j) bt[i * (size_t)MB + (size_t)j] = j < (int64_t)s->block_table.size() ? s->block_table[(size_t)j] : -1;
+        if (!want) wnt[i] = (int32_t)t - 1;
+    }
+    cu[nseq] = (int32_t)t;
+    if (want) for (size_t i = 0; i < R; ++i) { if (want[i] < 0 || want[i] >= T) return fail(NVR_ERR_INVALID_ARG, "execute_model: logits row %d of a step of %ld rows", want[i], (long)T); wnt[i] = want[i]; }
+    NVR_HIP_CHECK(hipMemcpyAsync(in_dev, in_host, off, hipMemcpyHostToDevice, r.stream));
+    kl::Batch b{};
+    b.ids = (const int64_t *)(in_dev + o_ids); b.row_seq = (const int32_t *)(in_dev + o_rs); b.cu = (const int32_t *)(in_dev + o_cu);
+    b.start = (const int32_t *)(in_dev + o_st); b.slot = (const int32_t *)(in_dev + o_sl); b.par = (const int32_t *)(in_dev + o_par);
+    b.block_tables = (const int32_t *)(in_dev + o_bt); b.max_blocks = (int32_t)MB; b.block_size = (int32_t)r.block_size;
+    b.T = (int32_t)T; b.B = (int32_t)nseq; b.max_ctx = (int32_t)max_ctx; b.max_rows = (int32_t)max_rows;
+    const int32_t *d_want = (const int32_t *)(in_dev + o_want);
+
+    hipStream_t s = r.stream;
+    const int64_t W = spec.width;
+    const float eps = (float)spec.eps;
+    RC(kl::embed_scale(embed, bf16, b.ids, T, W, (float)spec.embedding_scale, x, s));
+    for (size_t ri = 0; ri < spec.runs.size(); ++ri) {
+        const size_t li = (size_t)spec.runs[ri];
+        const LayeredSpec::Layer &L = spec.layers[li]; const LayerW &w = lw[li]; RunState &st = rs[ri];
+        RC(kl::norm_canon(x, b, W, eps, (int)spec.taps, w.g1, w.canon1, a1, w.g2, w.canon2, L.has_mlp ? a2 : nullptr, bf16, st.hist, slots, s));
+        RC(gemm(r, a1, W, w.mix, T, W, w.nmix, proj));
+        if (L.mixer == LayeredSpec::ATTENTION) {
+            RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, s));
+            kl::SinkAttnArgs a{};
+            a.q = proj + w.qcol; a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
+            a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
+            a.out = cat; a.ldo = w.kcat;
+            RC(kl::sink_attention(a, b, bf16, s));
+        } else {
+            kl::RetentionArgs a{};
+            a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.freq = w.freq; a.rot_dims = (int32_t)L.rot_dims;
+            a.kscale = 1.0f / std::sqrt((float)L.dim); a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.state = st.state; a.o = ret_o;
+            RC(kl::retention(a, b, s));
+            RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, cat, w.kcat, bf16, s));
+        }
+        if (L.has_mlp) {
+            RC(gemm(r, a2, W, w.gu, T, W, 2 * L.ff, gu));
+            RC(kl::clamped_glu(gu, T, L.ff, (float)L.limit, 1.702f, (char *)cat + (size_t)(w.mixcols * esz), w.kcat, bf16, s));
+        }
+        RC(gemm(r, cat, w.kcat, w.out, T, w.kcat, W, tmp));
+        RC(kl::axpy(x, tmp, (float)spec.residual_mult, T * W, s));
+    }
+    RC(kl::norm_rows(x, d_want, (int64_t)R, W, eps, gfinal, xsel, bf16, s));
+    RC(gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits));
+    for (size_t i = 0; i < nseq; ++i) slot_par[(size_t)seqs[i]->state_slot] ^= 1;
+    r.last_rows = R; r.last_tokens = T;
+    return NVR_OK;
+}
+
+}  // namespace nvr

@@ -1,0 +1,169 @@
+// model_registry.cpp — architecture name of a configuration file -> the model family that runs it and that family's description.
+// Dense decoder graphs (Qwen3Config, reference src/models/qwen3.rs:26-125) fill an nvr_model_config; layer-list designs fill a LayeredSpec.
+#include <cmath>
+#include <cstring>
+#include "common.h"
+#include "layered_model.h"
+
+namespace nvr {
+
+namespace {
+
+struct Reader {                                            // typed access with the path of the key in the error text
+    std::string err;
+    const Json *need(const Json &o, const char *key, const std::string &where) {
+        const Json *v = o.get(key);
+        if (!v && err.empty()) err = "config: '" + where + key + "' is missing";
+        return v;
+    }
+    double num(const Json &o, const char *key, const std::string &where) {
+        const Json *v = need(o, key, where);
+        if (!v) return 0;
+        if (v->kind != Json::Num) { if (err.empty()) err = "config: '" + where + key + "' is not a number"; return 0; }
+        return v->num;
+    }
+    int64_t integer(const Json &o, const char *key, const std::string &where) {
+        const double d = num(o, key, where);
+        if (d != std::floor(d) && err.empty()) err = "config: '" + where + key + "' is not an integer";
+        return (int64_t)d;
+    }
+};
+
+int parse_qwen3(const Json &c, nvr_model_spec *out) {
+    nvr_model_config &m = out->dense;
+    nvr_model_config_default(&m);
+    Reader rd;
+    m.vocab_size = (uint64_t)rd.integer(c, "vocab_size", ""); m.hidden_size = (uint64_t)rd.integer(c, "hidden_size", "");
+    m.intermediate_size = (uint64_t)rd.integer(c, "intermediate_size", ""); m.num_hidden_layers = (uint64_t)rd.integer(c, "num_hidden_layers", "");
+    m.num_attention_heads = (uint64_t)rd.integer(c, "num_attention_heads", "");
+    if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+    auto opt = [&](const char *k, double d) { const Json *v = c.get(k); return v && v->kind == Json::Num ? v->num : d; };
+    auto flag = [&](const char *k, bool d) { const Json *v = c.get(k); return v && v->kind == Json::Bool ? v->b : d; };
+    m.num_key_value_heads = (uint64_t)opt("num_key_value_heads", (double)m.num_attention_heads);
+    m.head_dim = (uint64_t)opt("head_dim", 0);
+    m.max_position_embeddings = (uint64_t)opt("max_position_embeddings", 32768);
+    m.rms_norm_eps = (float)opt("rms_norm_eps", 1e-6); m.rope_theta = opt("rope_theta", 10000.0);
+    m.tie_word_embeddings = flag("tie_word_embeddings", false);
+    m.qk_norm = flag("qk_norm", true);                      // checkpoints of this architecture carry q_norm / k_norm
+    m.use_bias = flag("attention_bias", false);
+    out->family = 0;
+    return NVR_OK;
+}
+
+int parse_rugudra_spec(const Json &c, nvr_model_spec *out) {
+    out->family = 1;
+    return LayeredSpec::parse_rugudra(c, &out->layered);
+}
+
+struct Entry { const char *name; int (*parse)(const Json &, nvr_model_spec *); };
+const Entry kRegistry[] = {
+    {"Qwen3ForCausalLM", parse_qwen3},
+    {"Rugudra", parse_rugudra_spec},
+};
+
+}  // namespace
+
+// Rugudra: every sublayer reads norm(x) through a short causal convolution; the mixer is softmax attention with a logarithmic distance
+// penalty and a sink, or retention; x <- x + m * (mixer + feed-forward); a range of layers may run several times.
+int LayeredSpec::parse_rugudra(const Json &c, LayeredSpec *s) {
+    Reader rd;
+    s->vocab = rd.integer(c, "vocab", ""); s->width = rd.integer(c, "width", "");
+    s->residual_mult = rd.num(c, "residual_mult", "");
+    if (const Json *e = rd.need(c, "embedding", "")) s->embedding_scale = rd.num(*e, "scale", "embedding.");
+    if (const Json *n = rd.need(c, "norm", "")) s->eps = rd.num(*n, "eps", "norm.");
+    if (const Json *k = rd.need(c, "canon", "")) s->taps = rd.integer(*k, "taps", "canon.");
+    const Json *layers = rd.need(c, "layers", "");
+    if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+    if (layers->kind != Json::Arr || layers->arr.empty()) return fail(NVR_ERR_INVALID_ARG, "config: 'layers' is not a list of layers");
+    s->layers.clear();
+    for (size_t i = 0; i < layers->arr.size(); ++i) {
+        const Json &lj = layers->arr[i];
+        const std::string w = "layers[" + std::to_string(i) + "].";
+        Layer L;
+        const Json *type = rd.need(lj, "type", w), *mx = rd.need(lj, "mixer", w);
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (type->kind != Json::Str) return fail(NVR_ERR_INVALID_ARG, "config: '%stype' is not a string", w.c_str());
+        L.heads = rd.integer(*mx, "heads", w + "mixer."); L.dim = rd.integer(*mx, "dim", w + "mixer."); L.vdim = rd.integer(*mx, "vdim", w + "mixer.");
+        if (type->str == "attention") {
+            L.mixer = ATTENTION;
+            L.kv_heads = rd.integer(*mx, "kv_heads", w + "mixer."); L.scale = rd.num(*mx, "scale", w + "mixer.");
+        } else if (type->str == "retention") {
+            L.mixer = RETENTION; L.kv_heads = L.heads;
+            const Json *d = rd.need(*mx, "decay", w + "mixer.");
+            if (d) {
+                if (d->kind != Json::Arr) return fail(NVR_ERR_INVALID_ARG, "config: '%smixer.decay' is not a list", w.c_str());
+                for (const Json &v : d->arr) L.decay.push_back(v.num);
+            }
+            const Json *rot = mx->get("rot");
+            if (rot && !rot->is_null()) { L.rot_dims = rd.integer(*rot, "dims", w + "mixer.rot."); L.rot_base = rd.num(*rot, "base", w + "mixer.rot."); }
+        } else return fail(NVR_ERR_UNSUPPORTED, "config: layer type '%s' (attention or retention)", type->str.c_str());
+        const Json *mlp = lj.get("mlp");
+        if (mlp && !mlp->is_null()) {
+            const Json *kind = mlp->get("kind");
+            if (kind && !(kind->kind == Json::Str && kind->str == "dense")) return fail(NVR_ERR_UNSUPPORTED, "config: '%smlp.kind' (dense)", w.c_str());
+            L.has_mlp = true; L.ff = rd.integer(*mlp, "ff", w + "mlp."); L.limit = rd.num(*mlp, "limit", w + "mlp.");
+        }
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (L.heads < 1 || L.dim < 1 || L.vdim < 1 || L.kv_heads < 1 || L.heads % L.kv_heads)
+            return fail(NVR_ERR_INVALID_ARG, "config: %s %ld heads over %ld key/value heads of %ld / %ld", w.c_str(), (long)L.heads, (long)L.kv_heads, (long)L.dim, (long)L.vdim);
+        if (L.mixer == RETENTION && ((int64_t)L.decay.size() != L.heads || L.rot_dims % 2 || L.rot_dims > L.dim || L.rot_dims < 0))
+            return fail(NVR_ERR_INVALID_ARG, "config: %s needs one decay per head and an even number of rotated coordinates <= dim", w.c_str());
+        if (L.has_mlp && L.ff < 1) return fail(NVR_ERR_INVALID_ARG, "config: '%smlp.ff' must be positive", w.c_str());
+        s->layers.push_back(L);
+    }
+    const int64_t n = (int64_t)s->layers.size();
+    s->runs.clear();
+    const Json *loop = c.get("loop");
+    if (loop && !loop->is_null()) {
+        const int64_t a = rd.integer(*loop, "start", "loop."), b = rd.integer(*loop, "stop", "loop."), t = rd.integer(*loop, "times", "loop.");
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (a < 0 || b < a || b > n || t < 1) return fail(NVR_ERR_INVALID_ARG, "config: loop [%ld, %ld) x %ld over %ld layers", (long)a, (long)b, (long)t, (long)n);
+        for (int64_t i = 0; i < a; ++i) s->runs.push_back((int)i);
+        for (int64_t k = 0; k < t; ++k) for (int64_t i = a; i < b; ++i) s->runs.push_back((int)i);
+        for (int64_t i = b; i < n; ++i) s->runs.push_back((int)i);
+    } else
+        for (int64_t i = 0; i < n; ++i) s->runs.push_back((int)i);
+    if (s->vocab < 1 || s->width < 1 || s->taps < 1) return fail(NVR_ERR_INVALID_ARG, "config: vocab, width and canon.taps must be positive");
+    return NVR_OK;
+}
+
+}  // namespace nvr
+
+extern "C" {
+
+size_t nvr_model_registry_size(void) { return sizeof(nvr::kRegistry) / sizeof(nvr::kRegistry[0]); }
+const char *nvr_model_registry_name(size_t i) { return i < nvr_model_registry_size() ? nvr::kRegistry[i].name : nullptr; }
+
+nvr_model_spec_t *nvr_model_spec_from_json(const char *text) {
+    try {
+        if (!text) { nvr::fail(NVR_ERR_INVALID_ARG, "config: no text"); return nullptr; }
+        nvr::Json c; std::string err;
+        if (!nvr::Json::parse(text, &c, &err)) { nvr::fail(NVR_ERR_INVALID_ARG, "config: %s", err.c_str()); return nullptr; }
+        std::string arch;
+        if (const nvr::Json *a = c.get("architecture")) { if (a->kind == nvr::Json::Str) arch = a->str; }
+        if (arch.empty())
+            if (const nvr::Json *a = c.get("architectures")) if (a->kind == nvr::Json::Arr && !a->arr.empty() && a->arr[0].kind == nvr::Json::Str) arch = a->arr[0].str;
+        if (arch.empty()) { nvr::fail(NVR_ERR_INVALID_ARG, "config: no 'architecture' (or 'architectures') entry"); return nullptr; }
+        for (const auto &e : nvr::kRegistry)
+            if (arch == e.name) {
+                std::unique_ptr<nvr_model_spec> sp(new nvr_model_spec());
+                sp->arch = arch;
+                if (e.parse(c, sp.get()) != NVR_OK) return nullptr;
+                return sp.release();
+            }
+        nvr::fail(NVR_ERR_UNSUPPORTED, "config: architecture '%s' is not registered", arch.c_str());
+        return nullptr;
+    } catch (...) { nvr::fail(NVR_ERR_INVARIANT, "config: out of memory"); return nullptr; }
+}
+void nvr_model_spec_destroy(nvr_model_spec_t *s) { delete s; }
+const char *nvr_model_spec_architecture(const nvr_model_spec_t *s) { return s->arch.c_str(); }
+int32_t nvr_model_spec_family(const nvr_model_spec_t *s) { return s->family; }
+int nvr_model_spec_dense(const nvr_model_spec_t *s, nvr_model_config *out) {
+    if (s->family != 0) return nvr::fail(NVR_ERR_INVALID_ARG, "architecture '%s' is not a dense graph", s->arch.c_str());
+    *out = s->dense;
+    return NVR_OK;
+}
+uint64_t nvr_model_spec_vocab(const nvr_model_spec_t *s) { return s->family == 0 ? s->dense.vocab_size : (uint64_t)s->layered.vocab; }
+uint64_t nvr_model_spec_num_layer_runs(const nvr_model_spec_t *s) { return s->family == 0 ? s->dense.num_hidden_layers : (uint64_t)s->layered.runs.size(); }
+
+}  // extern "C"

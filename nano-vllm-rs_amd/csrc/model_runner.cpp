@@ -58,6 +58,7 @@ nvr_model_runner::~nvr_model_runner() {
 }
 
 int nvr_model_runner::init() {                                       // ModelRunner::new, :67-102
+    if (layered) return layered->init(*this);
     env = nvr::Env::read();                                          // the only place the runner looks at the environment
     tp = (int64_t)cfg.tensor_parallel_size; rank = (int64_t)cfg.tensor_parallel_rank;
     bf16 = std::strcmp(cfg.dtype, "bfloat16") == 0;                               // config.rs:51 (fp16 otherwise)
@@ -456,6 +457,7 @@ bool match_layer(const char *name, const char *suffix, int64_t *layer) {        
 
 int nvr_model_runner::load_tensor(const char *name_in, int dtype, const int64_t *shape, int ndim, const void *data) {
     NVR_HIP_CHECK(hipSetDevice(device));
+    if (layered) { if (!name_in || !data || ndim < 0 || ndim > 2 || (ndim && !shape)) return nvr::fail(NVR_ERR_INVALID_ARG, "load_tensor: bad arguments"); return layered->load_tensor(*this, name_in, dtype, shape, ndim, data); }
     if (!name_in || !shape || !data || ndim < 1 || ndim > 2) return nvr::fail(NVR_ERR_INVALID_ARG, "load_tensor: bad arguments");
     if (dtype < 0 || dtype > 2) return nvr::fail(NVR_ERR_INVALID_ARG, "load_tensor: dtype %d (0 = f16, 1 = bf16, 2 = f32)", dtype);
     tiled_dirty = true;                                                   // the tiled copies are rebuilt before the next step
@@ -547,6 +549,7 @@ int nvr_model_runner::load_tensor(const char *name_in, int dtype, const int64_t 
 }
 
 int nvr_model_runner::copy_weight(const char *ln, uint16_t *out, size_t cap, int64_t *rows, int64_t *cols) {
+    if (layered) return nvr::fail(NVR_ERR_UNSUPPORTED, "copy_weight: not available for layer-list models");
     NVR_HIP_CHECK(hipSetDevice(device));
     const uint16_t *src = nullptr; int64_t r = 0, c = 0, l = -1;
     if (!std::strcmp(ln, "embed")) { src = embed; r = V; c = Hd; }
@@ -906,6 +909,10 @@ int nvr_model_runner::forward(int64_t T, int64_t B, bool is_prefill, int64_t max
 // execute_model :105-128 with prepare_*_inputs :172-210 and create_*_context :222-300
 int nvr_model_runner::execute(nvr_seq *const *seqs, size_t nseq, bool is_prefill) {
     NVR_HIP_CHECK(hipSetDevice(device));
+    if (layered) {                                                      // one step form for prompts, portions of prompts and decoded tokens
+        facts_shown_valid = false; last_prefill = is_prefill; lm_parts = 0; logits_valid = true;
+        return layered->execute(*this, seqs, nseq, nullptr, 0);
+    }
     if (tiled_dirty) RC(retile_all());
     if (tp > 1) RC(comm.prepare());
     if (tp > 1 && !comm.active() && !allow_missing_comm)
@@ -1395,7 +1402,7 @@ int nvr_model_runner::comm_selftest() {
 // the f32 logits of the last step, if that step skipped their stores: the LM-head launch is repeated on the same
 // (still resident) hidden rows with the stores on — same kernel, same bits
 int nvr_model_runner::ensure_logits() {
-    if (logits_valid) return NVR_OK;
+    if (logits_valid || layered) return NVR_OK;
     NVR_HIP_CHECK(hipSetDevice(device));
     int32_t np = 0;
     RC(KD(lm_head(lm_input, Hd, lm_head, (int64_t)last_rows, Hd, Vl, logits, d_lm_pval, d_lm_pidx, &np, stream, true,

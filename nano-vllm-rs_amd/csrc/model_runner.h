@@ -13,11 +13,14 @@
 #include "comm.h"
 #include "common.h"
 #include "kernels/kernels.h"
+#include "layered_model.h"
+#include <memory>
 
 struct nvr_model_runner {
     nvr::Env env;                          // NVR_* switches, read once in init()
     nvr_config cfg{};
     nvr_model_config mc{};
+    std::unique_ptr<nvr::LayeredModel> layered;   // set: a layer-list model (layered_model.cpp) runs the steps; the dense graph below is unused
     // derived, per rank (qwen3.rs:158-159, linear.rs:300-304)
     int64_t tp = 1, rank = 0;
     bool bf16 = false;                     // Config.dtype == "bfloat16": the nvr::kb build of the kernels; 16-bit words are bfloat16 everywhere
@@ -134,6 +137,7 @@ struct nvr_model_runner {
     uint16_t *v_cache(size_t l) { return kv_pool + (2 * l + 1) * kv_layer_elems * em; }
 
 private:
+    friend class nvr::LayeredModel;
     int forward(int64_t T, int64_t B, bool is_prefill, int64_t max_ctx);
     int gen_weights();
     int gen_weights_f32();

@@ -92,8 +92,24 @@ void nvr_seq_append_token(nvr_seq_t *s, int64_t t) { s->append_token(t); }
 int nvr_seq_should_stop(const nvr_seq_t *s, int has_eos, int64_t eos) { return s->should_stop(has_eos != 0, eos) ? 1 : 0; }
 void nvr_seq_preempt(nvr_seq_t *s) { s->preempt(); }
 void nvr_seq_finish(nvr_seq_t *s) { s->status = NVR_SEQ_FINISHED; }
+void nvr_seq_extend(nvr_seq_t *s, const int64_t *tokens, size_t n) { for (size_t i = 0; i < n; ++i) s->append_token(tokens[i]); }
+int nvr_seq_set_chunk(nvr_seq_t *s, size_t start, size_t len) {
+    if (len == 0 || start + len > s->num_tokens) return nvr::fail(NVR_ERR_INVALID_ARG, "set_chunk: [%zu, %zu) of a sequence of %zu tokens", start, start + len, s->num_tokens);
+    s->chunk_start = start; s->chunk_len = len;
+    return NVR_OK;
+}
+int32_t nvr_seq_state_slot(const nvr_seq_t *s) { return s->state_slot; }
 
 // ------------------------------------------------------------------ BlockManager
+nvr_block_manager_t *nvr_bm_create_stateful(size_t num_blocks, size_t block_size, size_t state_slots) {
+    NVR_GUARD_BEGIN
+    if (block_size == 0) { nvr::fail(NVR_ERR_INVALID_ARG, "Block size must be positive"); return nullptr; }
+    return new nvr_block_manager(num_blocks, block_size, state_slots);
+    NVR_GUARD_END(nullptr)
+}
+int nvr_bm_can_extend(const nvr_block_manager_t *bm, const nvr_seq_t *s) { return bm->impl.can_extend(*s) ? 1 : 0; }
+int nvr_bm_extend(nvr_block_manager_t *bm, nvr_seq_t *s) { NVR_GUARD_BEGIN return bm->impl.extend(*s); NVR_GUARD_END(NVR_ERR_INVARIANT) }
+size_t nvr_bm_free_state_slots(const nvr_block_manager_t *bm) { return bm->impl.free_state_slots(); }
 nvr_block_manager_t *nvr_bm_create(size_t num_blocks, size_t block_size) {
     if (num_blocks == 0) { nvr::fail(NVR_ERR_INVARIANT, "Number of blocks must be positive"); return nullptr; }   // :92
     if (block_size == 0) { nvr::fail(NVR_ERR_INVARIANT, "Block size must be positive"); return nullptr; }         // :93
@@ -169,6 +185,28 @@ nvr_model_runner_t *nvr_runner_create(const nvr_config *cfg, const nvr_model_con
     NVR_GUARD_END(nullptr)
 }
 void nvr_runner_destroy(nvr_model_runner_t *r) { delete r; }
+nvr_model_runner_t *nvr_runner_create_spec(const nvr_config *cfg, const nvr_model_spec_t *spec) {
+    NVR_GUARD_BEGIN
+    if (!spec) { nvr::fail(NVR_ERR_INVALID_ARG, "runner: no model description"); return nullptr; }
+    if (spec->family == 0) return nvr_runner_create(cfg, &spec->dense);
+    if (nvr_config_validate(cfg) || nvr_config_runnable(cfg)) return nullptr;
+    nvr_model_runner *r = new nvr_model_runner();
+    r->cfg = *cfg;
+    r->layered.reset(new nvr::LayeredModel());
+    r->layered->spec = spec->layered;
+    if (r->init() != NVR_OK) { delete r; return nullptr; }
+    return r;
+    NVR_GUARD_END(nullptr)
+}
+int nvr_runner_execute_step(nvr_model_runner_t *r, nvr_seq_t *const *seqs, size_t n, const int32_t *want_rows, size_t n_want, const float **logits_dev) {
+    NVR_GUARD_BEGIN
+    if (!r->layered) return nvr::fail(NVR_ERR_UNSUPPORTED, "execute_step: the dense graph's steps are prefill or decode (nvr_runner_execute_model)");
+    r->facts_shown_valid = false; r->last_prefill = true;
+    int rc = r->layered->execute(*r, seqs, n, want_rows, want_rows ? n_want : 0);
+    if (rc == NVR_OK && logits_dev) *logits_dev = r->logits;
+    return rc;
+    NVR_GUARD_END(NVR_ERR_INVARIANT)
+}
 int nvr_runner_execute_model(nvr_model_runner_t *r, nvr_seq_t *const *seqs, size_t n, int is_prefill, const float **logits_dev) {
     NVR_GUARD_BEGIN
     int rc = r->execute(seqs, n, is_prefill != 0);
@@ -199,6 +237,10 @@ int nvr_runner_copy_logits(nvr_model_runner_t *r, float *host_out, size_t rows) 
 uint64_t nvr_runner_num_kvcache_blocks(const nvr_model_runner_t *r) { return (uint64_t)r->num_blocks; }
 int nvr_runner_kv_cache(nvr_model_runner_t *r, size_t layer, void **kd, void **vd) {
     if ((int64_t)layer >= r->L) return nvr::fail(NVR_ERR_INVALID_ARG, "layer %zu out of range", layer);
+    if (r->layered) {                                                   // per layer RUN; a retention run has no pages (null)
+        *kd = r->layered->rs[layer].kc; *vd = r->layered->rs[layer].vc;
+        return NVR_OK;
+    }
     *kd = r->k_cache(layer); *vd = r->v_cache(layer);
     return NVR_OK;
 }
@@ -282,6 +324,25 @@ int nvr_runner_init_comm_local(nvr_model_runner_t *r, nvr_local_group_t *g) {
 }
 
 // ------------------------------------------------------------------ Engine
+nvr_engine_t *nvr_engine_create_spec(const nvr_config *cfg_in, const nvr_model_spec_t *spec) {
+    NVR_GUARD_BEGIN
+    if (!spec) { nvr::fail(NVR_ERR_INVALID_ARG, "engine: no model description"); return nullptr; }
+    if (spec->family == 0) return nvr_engine_create(cfg_in, &spec->dense);
+    nvr_config cfg = *cfg_in;
+    if (cfg.num_state_slots == 0) cfg.num_state_slots = cfg.max_num_seqs;      // one slot of state per sequence that can be live
+    cfg.async_decode = 0;                                                     // (launch-ahead rides on the dense graph's fused LM head)
+    if (nvr_config_validate(&cfg) || nvr_config_runnable(&cfg)) return nullptr;
+    std::unique_ptr<nvr_engine> e(new nvr_engine());
+    e->cfg = cfg;
+    e->runner.reset(nvr_runner_create_spec(&cfg, spec));
+    if (!e->runner) return nullptr;
+    nvr_config sc = cfg;
+    sc.num_kvcache_blocks = (int64_t)e->runner->num_blocks;
+    e->scheduler.reset(new nvr_scheduler(sc));
+    e->trace.on = e->runner->env.trace_host;
+    return e.release();
+    NVR_GUARD_END(nullptr)
+}
 nvr_engine_t *nvr_engine_create(const nvr_config *cfg, const nvr_model_config *mc) {
     NVR_GUARD_BEGIN
     if (nvr_config_validate(cfg) || nvr_config_runnable(cfg)) return nullptr;

@@ -9,7 +9,7 @@ Scheduler::Scheduler(const nvr_config &cfg)
     : max_num_seqs_(cfg.max_num_seqs), max_num_batched_tokens_(cfg.max_num_batched_tokens),
       has_eos_(cfg.has_eos != 0), eos_(cfg.eos_token_id), chunked_(cfg.enable_chunked_prefill != 0),
       bm_(new nvr_block_manager(cfg.num_kvcache_blocks >= 0 ? (size_t)cfg.num_kvcache_blocks : 1000,  // :71-74
-                                cfg.kvcache_block_size)) {}
+                                cfg.kvcache_block_size, (size_t)cfg.num_state_slots)) {}
 
 Scheduler::~Scheduler() {
     for (auto *s : waiting_) delete s;

@@ -23,6 +23,9 @@ struct nvr_seq {
     // chunked prefill (extension A-23; the reference schedules whole sequences, scheduler.rs:135-138): tokens whose K/V are in
     // the cache, and the token range [chunk_start, chunk_start + chunk_len) the sequence contributes to the step it is in
     size_t num_computed_tokens = 0, chunk_start = 0, chunk_len = 0;
+    // models with per-sequence state beside the K/V pages (recurrent state, convolution history): the slot the block manager gave this sequence
+    // together with its blocks (-1: none)
+    int32_t state_slot = -1;
     bool chunk_is_partial() const { return chunk_start + chunk_len < num_tokens; }
 
     size_t len() const { return num_tokens; }                                        // :104
@@ -47,7 +50,7 @@ struct nvr_seq {
         if (!sampling.ignore_eos && has_eos && last_token == eos) return true;
         return false;
     }
-    void preempt() { status = NVR_SEQ_PREEMPTED; block_table.clear(); num_cached_tokens = 0; num_computed_tokens = 0; chunk_start = chunk_len = 0; }  // :213
+    void preempt() { status = NVR_SEQ_PREEMPTED; block_table.clear(); state_slot = -1; num_cached_tokens = 0; num_computed_tokens = 0; chunk_start = chunk_len = 0; }  // :213
 };
 
 namespace nvr {
