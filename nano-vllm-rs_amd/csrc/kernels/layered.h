@@ -32,16 +32,16 @@ int embed_scale(const void *E, bool bf16, const int64_t *ids, int64_t T, int64_t
 int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, float g1, const float *w1, void *out1, float g2, const float *w2, void *out2,
                bool bf16, float *hist, int64_t slots, hipStream_t s);
 
-// rows of K ([G][D]) and V ([G][Dv]) out of the f32 projection rows (row stride ld; column offsets kcol / vcol) into the paged caches
+// rows of K ([G][D]) and V ([G][Dv]) out of the projection rows (operand type) (row stride ld; column offsets kcol / vcol) into the paged caches
 // [blocks][block_size][G][D] / [..][Dv] at the rows' positions
-int kv_store(const float *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
+int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
              hipStream_t s);
 
 // Causal softmax attention through the block tables: query row t at position i sees keys j <= i of its sequence;
 // score = q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)); the denominator also holds exp(sink[h]) (no key, no value).  r1 / r2 / sink may be null (plain
-// softmax attention).  q: f32 rows (stride ldq, heads [H][D]); out rows (stride ldo elements, heads [H][Dv]) of the operand type.
+// softmax attention).  q: rows of the operand type (stride ldq, heads [H][D]); out rows (stride ldo elements, heads [H][Dv]) of the operand type.
 struct SinkAttnArgs {
-    const float *q; int64_t ldq;
+    const void *q; int64_t ldq;             // operand type
     const void *kc, *vc;
     const float *r1, *r2, *sink;
     int32_t H, G, D, Dv; float scale;
@@ -50,29 +50,29 @@ struct SinkAttnArgs {
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);
 
 // Retention over the rows of a step: per head S <- decay[h] * S + k v^T, o = S^T q, with q and k rotated (first rot_dims coordinates, pairs (i, i + rot_dims/2),
-// angle = position * freq[i]) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: f32 rows (stride ld) holding
+// angle = position * freq[i]) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: rows of the operand type (stride ld) holding
 // q at column qcol ([H][D]), k at kcol, v at vcol ([H][Dv]).  o: f32 [T][H*Dv].
 struct RetentionArgs {
-    const float *proj; int64_t ld, qcol, kcol, vcol;
+    const void *proj; int64_t ld, qcol, kcol, vcol;
     const float *decay, *freq; int32_t rot_dims; float kscale;
     int32_t H, D, Dv;
     float *state; float *o;
 };
-int retention(const RetentionArgs &a, const Batch &b, hipStream_t s);
-// out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * silu(gate[t][h*Dv + c]); gate: f32 rows (stride ldg) from column gcol
-int head_norm_gate(const float *o, const float *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
+int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s);
+// out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * silu(gate[t][h*Dv + c]); gate: rows of the operand type (stride ldg) from column gcol
+int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
                    hipStream_t s);
 
-// g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gu: f32 rows [T][2*F] (gate columns, then up columns)
-int clamped_glu(const float *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s);
+// g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gu: rows [T][2*F] of the operand type (gate columns, then up columns)
+int clamped_glu(const void *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s);
 
-// x += mult * y (f32, [n])
-int axpy(float *x, const float *y, float mult, int64_t n, hipStream_t s);
+// x += mult * y (x f32, y of the operand type, [n])
+int axpy(float *x, const void *y, bool bf16, float mult, int64_t n, hipStream_t s);
 
 // out[r] = x[rows[r]] / sqrt(mean^2 + eps) * g, in the operand type
 int norm_rows(const float *x, const int32_t *rows, int64_t R, int64_t W, float eps, float g, void *out, bool bf16, hipStream_t s);
 
-// y[T][N] (f32) = a[T][K] . w[N][K]^T for shapes the tiled GEMMs do not take (any T, K, N)
-int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y, bool bf16, hipStream_t s);
+// y[T][N] (f32, or the operand type) = a[T][K] . w[N][K]^T for shapes the tiled GEMMs do not take (any T, K, N)
+int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32, bool bf16, hipStream_t s);
 
 }}  // namespace nvr::kl

@@ -118,15 +118,15 @@ __global__ __launch_bounds__(256) void norm_canon_kernel(const float *__restrict
 
 // ------------------------------------------------------------------------------------------------ K / V rows into the paged caches
 template <class CT>
-__global__ __launch_bounds__(256) void kv_store_kernel(const float *__restrict__ proj, int64_t ld, int64_t kcol, int64_t vcol, Batch b, int G, int D, int Dv,
+__global__ __launch_bounds__(256) void kv_store_kernel(const CT *__restrict__ proj, int64_t ld, int64_t kcol, int64_t vcol, Batch b, int G, int D, int Dv,
                                                        CT *__restrict__ kc, CT *__restrict__ vc) {
     const int t = blockIdx.x, sq = b.row_seq[t];
     const int p = b.start[sq] + (t - b.cu[sq]);
     const int blk = b.block_tables[(int64_t)sq * b.max_blocks + p / b.block_size];
     const int64_t row = (int64_t)blk * b.block_size + p % b.block_size;
-    const float *pr = proj + (int64_t)t * ld;
-    for (int c = threadIdx.x; c < G * D; c += 256) st_f(kc, row * G * D + c, pr[kcol + c]);
-    for (int c = threadIdx.x; c < G * Dv; c += 256) st_f(vc, row * G * Dv + c, pr[vcol + c]);
+    const CT *pr = proj + (int64_t)t * ld;
+    for (int c = threadIdx.x; c < G * D; c += 256) kc[row * G * D + c] = pr[kcol + c];
+    for (int c = threadIdx.x; c < G * Dv; c += 256) vc[row * G * Dv + c] = pr[vcol + c];
 }
 
 // ------------------------------------------------------------------------------------------------ attention with distance penalty and sink
@@ -139,8 +139,8 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
     const int i = b.start[sq] + (t - b.cu[sq]), ctx = i + 1;
     const int kvh = h / (a.H / a.G);
     float *qs = sm, *sc = sm + a.D;
-    const float *q = a.q + (int64_t)t * a.ldq + (int64_t)h * a.D;
-    for (int d = threadIdx.x; d < a.D; d += 256) qs[d] = q[d];
+    const CT *q = (const CT *)a.q + (int64_t)t * a.ldq + (int64_t)h * a.D;
+    for (int d = threadIdx.x; d < a.D; d += 256) qs[d] = ld_f(q, d);
     __syncthreads();
     const CT *kc = (const CT *)a.kc; const CT *vc = (const CT *)a.vc;
     const int32_t *bt = b.block_tables + (int64_t)sq * b.max_blocks;
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
 
 // ------------------------------------------------------------------------------------------------ retention, token by token
 // One workgroup per (sequence, head, block of 32 value columns): thread (c, part) keeps rows part, part + 8, ... of column c of the state in registers.
-template <int RMAX>
+template <int RMAX, class PT>
 __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Batch b) {
     __shared__ float qs[2][512], ks[2][512], red[8][32];
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
@@ -199,21 +199,21 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
     for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
     for (int i = 0; i < n; ++i) {
         const int t = r0 + i, buf = i & 1;
-        const float *pr = a.proj + (int64_t)t * a.ld;
-        const float *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
+        const PT *pr = (const PT *)a.proj + (int64_t)t * a.ld;
+        const PT *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
         for (int d = threadIdx.x; d < D; d += 256) {
-            float qv = q[d], kv = k[d];
+            float qv = ld_f(q, d), kv = ld_f(k, d);
             if (d < a.rot_dims) {
                 const int fi = d < half ? d : d - half;
                 const float ang = (float)(st + i) * a.freq[fi];
                 float sn, cs; sincosf(ang, &sn, &cs);
-                if (d < half) { qv = qv * cs - q[d + half] * sn; kv = kv * cs - k[d + half] * sn; }
-                else { qv = qv * cs + q[d - half] * sn; kv = kv * cs + k[d - half] * sn; }
+                if (d < half) { qv = qv * cs - ld_f(q, d + half) * sn; kv = kv * cs - ld_f(k, d + half) * sn; }
+                else { qv = qv * cs + ld_f(q, d - half) * sn; kv = kv * cs + ld_f(k, d - half) * sn; }
             }
             qs[buf][d] = qv; ks[buf][d] = kv * a.kscale;
         }
         __syncthreads();
-        const float v = live ? pr[a.vcol + (int64_t)h * Dv + c] : 0.f;
+        const float v = live ? ld_f(pr, a.vcol + (int64_t)h * Dv + c) : 0.f;
         float o = 0.f;
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
 }
 
 template <class OT>
-__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float *__restrict__ o, const float *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float *__restrict__ o, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
                                                             float eps, OT *__restrict__ out, int64_t ldo) {
     const int64_t t = blockIdx.x; const int h = blockIdx.y;
     const float *orow = o + (t * H + h) * Dv;
@@ -245,24 +245,25 @@ __global__ __launch_bounds__(64) void head_norm_gate_kernel(const float *__restr
     ss = wave_sum(ss);
     const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
     for (int c = threadIdx.x; c < Dv; c += 64) {
-        const float g = gate[t * ldg + gcol + (int64_t)h * Dv + c];
+        const float g = ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c);
         st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (g / (1.0f + expf(-g))));
     }
 }
 
 template <class OT>
-__global__ __launch_bounds__(256) void clamped_glu_kernel(const float *__restrict__ gu, int64_t T, int64_t F, float limit, float alpha, OT *__restrict__ out, int64_t ldo) {
+__global__ __launch_bounds__(256) void clamped_glu_kernel(const OT *__restrict__ gu, int64_t T, int64_t F, float limit, float alpha, OT *__restrict__ out, int64_t ldo) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= T * F) return;
     const int64_t t = idx / F, c = idx - t * F;
-    const float g = fminf(gu[t * 2 * F + c], limit);
-    const float u = fminf(fmaxf(gu[t * 2 * F + F + c], -limit), limit);
+    const float g = fminf(ld_f(gu, t * 2 * F + c), limit);
+    const float u = fminf(fmaxf(ld_f(gu, t * 2 * F + F + c), -limit), limit);
     st_f(out, t * ldo + c, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
 }
 
-__global__ __launch_bounds__(256) void axpy_kernel(float *__restrict__ x, const float *__restrict__ y, float m, int64_t n) {
+template <class YT>
+__global__ __launch_bounds__(256) void axpy_kernel(float *__restrict__ x, const YT *__restrict__ y, float m, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) x[i] += m * y[i];
+    if (i < n) x[i] += m * ld_f(y, i);
 }
 
 template <class OT>
@@ -277,8 +278,8 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float *__restrict_
     for (int c = threadIdx.x; c < W; c += 256) st_f(out, r * W + c, xr[c] * rs * g);
 }
 
-template <class ET>
-__global__ __launch_bounds__(256) void gemm_any_kernel(const ET *__restrict__ a, int64_t lda, const ET *__restrict__ w, int T, int K, int N, float *__restrict__ y) {
+template <class ET, class YT>
+__global__ __launch_bounds__(256) void gemm_any_kernel(const ET *__restrict__ a, int64_t lda, const ET *__restrict__ w, int T, int K, int N, YT *__restrict__ y) {
     __shared__ float as[16][17], ws[16][17];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int t = blockIdx.y * 16 + ty, nn = blockIdx.x * 16 + tx;
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void gemm_any_kernel(const ET *__restrict__ a,
         for (int kk = 0; kk < 16; ++kk) acc += as[ty][kk] * ws[tx][kk];
         __syncthreads();
     }
-    if (t < T && nn < N) y[(int64_t)t * N + nn] = acc;
+    if (t < T && nn < N) st_f(y, (int64_t)t * N + nn, acc);
 }
 
 }  // namespace
@@ -326,11 +327,11 @@ int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, f
     return launched("norm_canon");
 }
 
-int kv_store(const float *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
+int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
              hipStream_t s) {
     if (b.T == 0) return 0;
-    if (bf16) kv_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (bf16_t *)kc, (bf16_t *)vc);
-    else kv_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>(proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (float *)kc, (float *)vc);
+    if (bf16) kv_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (bf16_t *)kc, (bf16_t *)vc);
+    else kv_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (float *)kc, (float *)vc);
     return launched("kv_store");
 }
 
@@ -345,39 +346,46 @@ int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t
     return launched("sink_attention");
 }
 
-int retention(const RetentionArgs &a, const Batch &b, hipStream_t s) {
+int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
     if (a.D > 512) return nvr::fail(NVR_ERR_UNSUPPORTED, "retention: key size %d (at most 512)", a.D);
     if (a.rot_dims % 2 || a.rot_dims > a.D) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: %d rotated coordinates of %d", a.rot_dims, a.D);
     const dim3 grid((unsigned)b.B, (unsigned)a.H, (unsigned)((a.Dv + 31) / 32));
     const int rows = (a.D + 7) / 8;
-    if (rows <= 8) retention_seq_kernel<8><<<grid, dim3(256), 0, s>>>(a, b);
-    else if (rows <= 16) retention_seq_kernel<16><<<grid, dim3(256), 0, s>>>(a, b);
-    else if (rows <= 32) retention_seq_kernel<32><<<grid, dim3(256), 0, s>>>(a, b);
-    else retention_seq_kernel<64><<<grid, dim3(256), 0, s>>>(a, b);
+#define NVR_RET(R_)                                                                                  \
+    do {                                                                                             \
+        if (bf16) retention_seq_kernel<R_, bf16_t><<<grid, dim3(256), 0, s>>>(a, b);                 \
+        else retention_seq_kernel<R_, float><<<grid, dim3(256), 0, s>>>(a, b);                       \
+    } while (0)
+    if (rows <= 8) NVR_RET(8);
+    else if (rows <= 16) NVR_RET(16);
+    else if (rows <= 32) NVR_RET(32);
+    else NVR_RET(64);
+#undef NVR_RET
     return launched("retention");
 }
 
-int head_norm_gate(const float *o, const float *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
+int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
                    hipStream_t s) {
     if (T == 0) return 0;
     const dim3 grid((unsigned)T, (unsigned)H);
-    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(64), 0, s>>>(o, gate, ldg, gcol, (int)H, (int)Dv, eps, (bf16_t *)out, ldo);
-    else head_norm_gate_kernel<float><<<grid, dim3(64), 0, s>>>(o, gate, ldg, gcol, (int)H, (int)Dv, eps, (float *)out, ldo);
+    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(64), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, (bf16_t *)out, ldo);
+    else head_norm_gate_kernel<float><<<grid, dim3(64), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, (float *)out, ldo);
     return launched("head_norm_gate");
 }
 
-int clamped_glu(const float *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s) {
+int clamped_glu(const void *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s) {
     if (T * F == 0) return 0;
     const dim3 grid((unsigned)((T * F + 255) / 256));
-    if (bf16) clamped_glu_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(gu, T, F, limit, alpha, (bf16_t *)out, ldo);
-    else clamped_glu_kernel<float><<<grid, dim3(256), 0, s>>>(gu, T, F, limit, alpha, (float *)out, ldo);
+    if (bf16) clamped_glu_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)gu, T, F, limit, alpha, (bf16_t *)out, ldo);
+    else clamped_glu_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)gu, T, F, limit, alpha, (float *)out, ldo);
     return launched("clamped_glu");
 }
 
-int axpy(float *x, const float *y, float mult, int64_t n, hipStream_t s) {
+int axpy(float *x, const void *y, bool bf16, float mult, int64_t n, hipStream_t s) {
     if (n == 0) return 0;
-    axpy_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(x, y, mult, n);
+    if (bf16) axpy_kernel<bf16_t><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(x, (const bf16_t *)y, mult, n);
+    else axpy_kernel<float><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(x, (const float *)y, mult, n);
     return launched("axpy");
 }
 
@@ -388,11 +396,12 @@ int norm_rows(const float *x, const int32_t *rows, int64_t R, int64_t W, float e
     return launched("norm_rows");
 }
 
-int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y, bool bf16, hipStream_t s) {
+int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32, bool bf16, hipStream_t s) {
     if (T == 0 || N == 0) return 0;
     const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((T + 15) / 16));
-    if (bf16) gemm_any_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)a, lda, (const bf16_t *)w, (int)T, (int)K, (int)N, y);
-    else gemm_any_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)a, lda, (const float *)w, (int)T, (int)K, (int)N, y);
+    if (bf16 && y_f32) gemm_any_kernel<bf16_t, float><<<grid, dim3(256), 0, s>>>((const bf16_t *)a, lda, (const bf16_t *)w, (int)T, (int)K, (int)N, (float *)y);
+    else if (bf16) gemm_any_kernel<bf16_t, bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)a, lda, (const bf16_t *)w, (int)T, (int)K, (int)N, (bf16_t *)y);
+    else gemm_any_kernel<float, float><<<grid, dim3(256), 0, s>>>((const float *)a, lda, (const float *)w, (int)T, (int)K, (int)N, (float *)y);
     return launched("gemm_any");
 }
 

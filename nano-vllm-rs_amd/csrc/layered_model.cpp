@@ -131,8 +131,8 @@ int LayeredModel::init(nvr_model_runner &r) {
 
     // activations
     const int64_t MT = r.max_tokens;
-    RC(dmalloc(&x, (size_t)(MT * W * 4))); RC(dmalloc(&tmp, (size_t)(MT * W * 4)));
-    RC(dmalloc(&proj, (size_t)(MT * max_nmix * 4))); RC(dmalloc(&gu, (size_t)(MT * 2 * max_ff * 4))); RC(dmalloc(&ret_o, (size_t)(MT * max_hv * 4)));
+    RC(dmalloc(&x, (size_t)(MT * W * 4))); RC(dmalloc(&tmp, (size_t)(MT * W * esz)));
+    RC(dmalloc(&proj, (size_t)(MT * max_nmix * esz))); RC(dmalloc(&gu, (size_t)(MT * 2 * max_ff * esz))); RC(dmalloc(&ret_o, (size_t)(MT * max_hv * 4)));
     RC(dmalloc(&a1, (size_t)(MT * W * esz))); RC(dmalloc(&a2, (size_t)(MT * W * esz))); RC(dmalloc(&cat, (size_t)(MT * max_kcat * esz)));
     logit_rows_cap = std::max<int64_t>(r.max_seqs, 64);
     RC(dmalloc(&xsel, (size_t)(std::max(MT, logit_rows_cap) * W * esz)));
@@ -217,10 +217,12 @@ int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtyp
     return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in);
 }
 
-int LayeredModel::gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y) {
-    if (!bf16) return nvr::kf::linear((const float *)a, lda, (const float *)w, T, K, N, nullptr, y, r.stream);
-    if (K % 32 == 0 && N % 16 == 0 && lda % 8 == 0) return nvr::kb::linear((const uint16_t *)a, lda, (const uint16_t *)w, T, K, N, y, true, r.stream);
-    return kl::gemm_any(a, lda, w, T, K, N, y, true, r.stream);
+// y = a . w^T in the operand type (bf16: f32 accumulation on the matrix cores, one rounding at the store; the dense graph's GEMM routing), or, for the
+// logits, in f32
+int LayeredModel::gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32) {
+    if (!bf16) return nvr::kf::linear((const float *)a, lda, (const float *)w, T, K, N, nullptr, (float *)y, r.stream);
+    if (K % 32 == 0 && N % 16 == 0 && lda % 8 == 0) return nvr::kb::linear((const uint16_t *)a, lda, (const uint16_t *)w, T, K, N, y, y_f32, r.stream);
+    return kl::gemm_any(a, lda, w, T, K, N, y, y_f32, true, r.stream);
 }
 
 // One step over a batch of chunks: sequence i contributes its tokens [chunk_start, chunk_start + chunk_len).  want: rows of the step (in batch
@@ -295,7 +297,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
         if (L.mixer == LayeredSpec::ATTENTION) {
             RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, s));
             kl::SinkAttnArgs a{};
-            a.q = proj + w.qcol; a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
+            a.q = (const char *)proj + (size_t)(w.qcol * esz); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
             a.out = cat; a.ldo = w.kcat;
             RC(kl::sink_attention(a, b, bf16, s));
@@ -303,7 +305,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
             kl::RetentionArgs a{};
             a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.freq = w.freq; a.rot_dims = (int32_t)L.rot_dims;
             a.kscale = 1.0f / std::sqrt((float)L.dim); a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.state = st.state; a.o = ret_o;
-            RC(kl::retention(a, b, s));
+            RC(kl::retention(a, b, bf16, s));
             RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, cat, w.kcat, bf16, s));
         }
         if (L.has_mlp) {
@@ -311,10 +313,10 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
             RC(kl::clamped_glu(gu, T, L.ff, (float)L.limit, 1.702f, (char *)cat + (size_t)(w.mixcols * esz), w.kcat, bf16, s));
         }
         RC(gemm(r, cat, w.kcat, w.out, T, w.kcat, W, tmp));
-        RC(kl::axpy(x, tmp, (float)spec.residual_mult, T * W, s));
+        RC(kl::axpy(x, tmp, bf16, (float)spec.residual_mult, T * W, s));
     }
     RC(kl::norm_rows(x, d_want, (int64_t)R, W, eps, gfinal, xsel, bf16, s));
-    RC(gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits));
+    RC(gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits, true));
     for (size_t i = 0; i < nseq; ++i) slot_par[(size_t)seqs[i]->state_slot] ^= 1;
     r.last_rows = R; r.last_tokens = T;
     return NVR_OK;

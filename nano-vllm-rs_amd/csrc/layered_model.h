@@ -55,8 +55,8 @@ public:
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;
     // activations
-    float *x = nullptr, *proj = nullptr, *gu = nullptr, *tmp = nullptr, *ret_o = nullptr;
-    void *a1 = nullptr, *a2 = nullptr, *cat = nullptr, *xsel = nullptr;
+    float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32
+    void *proj = nullptr, *gu = nullptr, *tmp = nullptr, *a1 = nullptr, *a2 = nullptr, *cat = nullptr, *xsel = nullptr;   // operand type
     int64_t slots = 0; std::vector<int32_t> slot_par;
     // step inputs
     char *in_host = nullptr, *in_dev = nullptr; size_t in_bytes = 0;
@@ -68,7 +68,7 @@ public:
     int load_tensor(nvr_model_runner &r, const char *name, int dtype, const int64_t *shape, int ndim, const void *data);
 
 private:
-    int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, float *y);
+    int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);
 };
 
