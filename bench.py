@@ -698,7 +698,18 @@ def main() -> None:
     ap.add_argument("--no-live-pmc", action="store_true",
                     help="do not run the child rocprofv3 --pmc FETCH_SIZE pass that counts roofline.traffic in this run (N = 1; "
                          "NVR_BENCH_LIVE_PMC=0 does the same): the committed pass under profiles/ is quoted instead")
+    ap.add_argument("--layered-compare", action="store_true",
+                    help="instead of the headline workload: prefill and decode throughput of a Rugudra-design model (attention with distance penalty and sink, "
+                         "retention, clamped gated feed-forward) beside the dense Qwen3 graph at equal layer sizes, random weights, one JSON line per size")
+    ap.add_argument("--layered-sizes", default="w1024,w2048", help="sizes of --layered-compare (w1024, w2048, w4096)")
+    ap.add_argument("--layered-models", default="rugudra,qwen3", help="models of --layered-compare")
     args = ap.parse_args()
+    if args.layered_compare:
+        import importlib
+        nvr = nvr_import.load()
+        lb = importlib.import_module(nvr.__name__ + ".layered_bench")
+        lb.compare(nvr, sizes=tuple(args.layered_sizes.split(",")), steps=min(args.steps, 32), warmup=min(args.warmup, 4), which=tuple(args.layered_models.split(",")))
+        return
     global BATCH, PROMPT_LEN
     BATCH, PROMPT_LEN = MODELS[args.model]["batch"], MODELS[args.model]["prompt_len"]
     # Control-plane dry runs of 4 / 8 rank PROCESSES on ONE GPU only (tools/tp_dryrun.sh, NRANKS >= 4): every cross-process rendezvous of a one-shot collective

@@ -47,7 +47,14 @@ struct SinkAttnArgs {
     int32_t H, G, D, Dv; float scale;
     void *out; int64_t ldo;
 };
-int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);
+int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
+// The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
+// rows row0 .. row0 + 64 / (H / G) - 1 of sequence seq's chunk, for all H / G query heads of a key/value head.  nsplit > 1 spreads a tile's keys over that many
+// workgroups (decode-sized steps over long contexts) and merges their partials; workspace: sink_attention_workspace_bytes(ntiles * G * nsplit).
+struct AttnTile { int32_t seq, row0; };
+bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16);
+size_t sink_attention_workspace_bytes(int max_workgroups);
+int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s);
 
 // Retention over the rows of a step: per head S <- decay[h] * S + k v^T, o = S^T q, with q and k rotated (first rot_dims coordinates, pairs (i, i + rot_dims/2),
 // angle = position * freq[i]) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: rows of the operand type (stride ld) holding

@@ -2,6 +2,7 @@
 // of each sublayer, attention with distance penalty and sink, retention with f32 state, clamped gated feed-forward.  wave64, gfx950.
 #include <hip/hip_runtime.h>
 #include <math.h>
+#include <algorithm>
 #include "../common.h"
 #include "layered.h"
 
@@ -182,6 +183,182 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
     }
 }
 
+// Matrix-core form (bf16 operands; D and Dv multiples of 32 / 16 up to the size class C).  A workgroup owns one tile — up to 64 / g consecutive
+// positions of one sequence times the g = H / G query heads of one key/value head, 16 rows per wave — and walks the keys in tiles of 64 through LDS:
+// S = Q K^T on v_mfma_f32_16x16x32_bf16, penalty / mask / online softmax in f32 on the accumulator layout (lane: key column, four rows), P rounded
+// to bf16 through LDS into the A layout, O += P V with V held transposed in LDS.  The sink starts the running maximum and counts 1 in the running
+// sum.  nsplit > 1: workgroup z takes every nsplit-th share of the keys and leaves (o, m, l) partials for sink_attn_merge_kernel.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int C>
+__global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, float *__restrict__ part_o,
+                                                             float *__restrict__ part_ml) {
+    constexpr int KT = 64, KS = C + 8, VS = KT + 8;
+    extern __shared__ char smem[];
+    bf16_t *Ks = (bf16_t *)smem;                        // [KT][KS] keys x dims
+    bf16_t *Vt = Ks + KT * KS;                          // [C][VS] value columns x keys
+    bf16_t *Ps = Vt + C * VS;                           // [4][16][VS] one wave's weights
+    const int tile = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+    const int sq = tiles[tile].seq, lr0 = tiles[tile].row0;
+    const int c0 = b.cu[sq], n = b.cu[sq + 1] - c0, st = b.start[sq];
+    const int g = a.H / a.G, PW = 64 / g;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4;
+    const int D = a.D, Dv = a.Dv, d32 = D >> 5, dv16 = Dv >> 4;
+    const int npos = min(PW, n - lr0);                  // positions of this tile
+    const bool wave_on = wave * 16 < npos * g;
+    const bf16_t *kc = (const bf16_t *)a.kc, *vc = (const bf16_t *)a.vc;
+    const int32_t *bt = b.block_tables + (int64_t)sq * b.max_blocks;
+
+    bf16x8 qf[C / 32];
+    {
+        const int r = wave * 16 + lm, pi = min(r / g, npos - 1), hg = r % g;
+        const bf16_t *q = (const bf16_t *)a.q + (int64_t)(c0 + lr0 + pi) * a.ldq + (int64_t)(kvh * g + hg) * D + lq * 8;
+#pragma unroll
+        for (int ks = 0; ks < C / 32; ++ks) if (ks < d32) qf[ks] = *reinterpret_cast<const bf16x8 *>(q + ks * 32);
+    }
+    int pos[4]; float r1[4], r2[4], m[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = wave * 16 + lq * 4 + i, h = kvh * g + r % g;
+        pos[i] = st + lr0 + r / g;
+        r1[i] = a.r1 ? a.r1[h] : 0.f; r2[i] = a.r2 ? a.r2[h] : 0.f;
+        const bool sink_here = a.sink && z == 0;
+        m[i] = sink_here ? a.sink[h] : -INFINITY;
+        l[i] = (sink_here && lm == 0) ? 1.f : 0.f;
+    }
+    f32x4 acc[C / 16];
+#pragma unroll
+    for (int t = 0; t < C / 16; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nkeys = st + lr0 + npos;                  // keys the tile's last position sees
+    const int ntl = (nkeys + KT - 1) / KT;
+    for (int kt = z; kt < ntl; kt += nsplit) {
+        const int k0 = kt * KT;
+        __syncthreads();
+        const int kch = D >> 3, vch = Dv >> 3;
+        for (int idx = threadIdx.x; idx < KT * kch; idx += 256) {
+            const int key = idx / kch, ch = idx - key * kch, j = k0 + key;
+            uint4 v = uint4{0, 0, 0, 0};
+            if (j < nkeys) {
+                const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
+                v = *reinterpret_cast<const uint4 *>(kc + (row * a.G + kvh) * D + ch * 8);
+            }
+            *reinterpret_cast<uint4 *>(Ks + key * KS + ch * 8) = v;
+        }
+        for (int idx = threadIdx.x; idx < KT * vch; idx += 256) {
+            const int ch = idx / KT, key = idx - ch * KT, j = k0 + key;      // (consecutive threads: consecutive keys of one column block)
+            uint4 v = uint4{0, 0, 0, 0};
+            if (j < nkeys) {
+                const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
+                v = *reinterpret_cast<const uint4 *>(vc + (row * a.G + kvh) * Dv + ch * 8);
+            }
+            const bf16_t *e = reinterpret_cast<const bf16_t *>(&v);
+#pragma unroll
+            for (int x = 0; x < 8; ++x) Vt[(ch * 8 + x) * VS + key] = e[x];
+        }
+        __syncthreads();
+        if (wave_on) {
+            f32x4 s[4];
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                s[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < C / 32; ++ks)
+                    if (ks < d32) {
+                        const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(Ks + (nt * 16 + lm) * KS + ks * 32 + lq * 8);
+                        s[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], kf, s[nt], 0, 0, 0);
+                    }
+            }
+            float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const int j = k0 + nt * 16 + lm;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = s[nt][i] * a.scale;
+                    if (a.r1) v -= r1[i] * __logf(1.0f + r2[i] * (float)(pos[i] - j));
+                    v = (j > pos[i]) ? -INFINITY : v;
+                    s[nt][i] = v;
+                    mx[i] = fmaxf(mx[i], v);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int o = 1; o < 16; o <<= 1) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], o, 64));
+                const float mn = fmaxf(m[i], mx[i]);
+                const float alpha = (m[i] == -INFINITY) ? 0.f : __expf(m[i] - mn);
+                m[i] = mn;
+                float rs = 0.f;
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const float p = (s[nt][i] == -INFINITY) ? 0.f : __expf(s[nt][i] - mn);
+                    rs += p;
+                    st_f(Ps, (wave * 16 + lq * 4 + i) * VS + nt * 16 + lm, p);
+                }
+                l[i] = l[i] * alpha + rs;
+#pragma unroll
+                for (int t = 0; t < C / 16; ++t) acc[t][i] *= alpha;
+            }
+        }
+        __syncthreads();
+        if (wave_on) {
+#pragma unroll
+            for (int k2 = 0; k2 < KT / 32; ++k2) {
+                const bf16x8 pf = *reinterpret_cast<const bf16x8 *>(Ps + (wave * 16 + lm) * VS + k2 * 32 + lq * 8);
+#pragma unroll
+                for (int t = 0; t < C / 16; ++t)
+                    if (t < dv16) {
+                        const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(Vt + (t * 16 + lm) * VS + k2 * 32 + lq * 8);
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc[t], 0, 0, 0);
+                    }
+            }
+        }
+    }
+    if (!wave_on) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) l[i] += __shfl_xor(l[i], o, 64);
+        const int r = wave * 16 + lq * 4 + i, pi = r / g, hg = r % g;
+        if (pi >= npos) continue;
+        if (nsplit == 1) {
+            const float inv = 1.0f / l[i];
+            bf16_t *o = (bf16_t *)a.out + (int64_t)(c0 + lr0 + pi) * a.ldo + (int64_t)(kvh * g + hg) * Dv;
+#pragma unroll
+            for (int t = 0; t < C / 16; ++t) if (t < dv16) st_f(o, t * 16 + lm, acc[t][i] * inv);
+        } else {
+            const int64_t pr = (((int64_t)tile * a.G + kvh) * nsplit + z) * 64 + r;
+#pragma unroll
+            for (int t = 0; t < C / 16; ++t) if (t < dv16) part_o[pr * Dv + t * 16 + lm] = acc[t][i];
+            if (lm == 0) { part_ml[pr * 2] = m[i]; part_ml[pr * 2 + 1] = l[i]; }
+        }
+    }
+}
+
+// one wave per (tile, key/value head, row): out = sum_z o_z e^(m_z - m) / sum_z l_z e^(m_z - m)
+__global__ __launch_bounds__(64) void sink_attn_merge_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, const float *__restrict__ part_o,
+                                                             const float *__restrict__ part_ml) {
+    const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
+    const int sq = tiles[tile].seq, lr0 = tiles[tile].row0;
+    const int c0 = b.cu[sq], n = b.cu[sq + 1] - c0;
+    const int g = a.H / a.G, PW = 64 / g, npos = min(PW, n - lr0);
+    const int pi = r / g, hg = r % g;
+    if (pi >= npos) return;
+    const int64_t base = ((int64_t)tile * a.G + kvh) * nsplit;
+    float m = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) m = fmaxf(m, part_ml[((base + z) * 64 + r) * 2]);
+    float l = 0.f;
+    for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) l += part_ml[((base + z) * 64 + r) * 2 + 1] * __expf(mz - m); }
+    bf16_t *o = (bf16_t *)a.out + (int64_t)(c0 + lr0 + pi) * a.ldo + (int64_t)(kvh * g + hg) * a.Dv;
+    for (int c = threadIdx.x; c < a.Dv; c += 64) {
+        float acc = 0.f;
+        for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) acc += part_o[((base + z) * 64 + r) * a.Dv + c] * __expf(mz - m); }
+        st_f(o, c, acc / l);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ retention, token by token
 // One workgroup per (sequence, head, block of 32 value columns): thread (c, part) keeps rows part, part + 8, ... of column c of the state in registers.
 template <int RMAX, class PT>
@@ -304,6 +481,9 @@ static const size_t kMaxLds = 160 * 1024 - 2048;
 int prepare() {
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_rows_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_rows_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
+    NVR_HIP_CHECK(hipFuncSetAttribute((const void *)sink_attn_mfma_kernel<256>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)norm_canon_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     NVR_HIP_CHECK(hipFuncSetAttribute((const void *)norm_canon_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds));
     return 0;
@@ -333,6 +513,36 @@ int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Bat
     if (bf16) kv_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (bf16_t *)kc, (bf16_t *)vc);
     else kv_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (float *)kc, (float *)vc);
     return launched("kv_store");
+}
+
+bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16) {
+    return bf16 && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
+           ((uintptr_t)a.q % 16) == 0 && ((uintptr_t)a.kc % 16) == 0 && ((uintptr_t)a.vc % 16) == 0;
+}
+size_t sink_attention_workspace_bytes(int max_workgroups) { return (size_t)max_workgroups * 64 * (256 + 2) * sizeof(float); }
+
+int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    if (ntiles == 0) return 0;
+    if (!sink_attention_tiled_ok(a, true)) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention_tiled: shape outside the matrix-core kernel");
+    if (nsplit < 1) nsplit = 1;
+    float *po = nullptr, *pml = nullptr;
+    if (nsplit > 1) {
+        const size_t rows = (size_t)ntiles * a.G * nsplit * 64;
+        if (rows * (a.Dv + 2) * sizeof(float) > workspace_bytes) return nvr::fail(NVR_ERR_INVALID_ARG, "sink_attention_tiled: workspace too small for %d splits", nsplit);
+        po = (float *)workspace; pml = po + rows * a.Dv;
+    }
+    const int C = std::max(a.D, a.Dv) <= 64 ? 64 : std::max(a.D, a.Dv) <= 128 ? 128 : 256;
+    const size_t lds = ((size_t)64 * (C + 8) + (size_t)C * 72 + (size_t)64 * 72) * 2;
+    const dim3 grid((unsigned)ntiles, (unsigned)a.G, (unsigned)nsplit);
+    if (C == 64) sink_attn_mfma_kernel<64><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+    else if (C == 128) sink_attn_mfma_kernel<128><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+    else sink_attn_mfma_kernel<256><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
+    if (int rc = launched("sink_attention_tiled")) return rc;
+    if (nsplit > 1) {
+        sink_attn_merge_kernel<<<dim3((unsigned)ntiles, (unsigned)a.G, 64), dim3(64), 0, s>>>(a, b, tiles, nsplit, po, pml);
+        return launched("sink_attention merge");
+    }
+    return 0;
 }
 
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s) {

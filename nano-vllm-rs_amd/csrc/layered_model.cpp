@@ -42,6 +42,7 @@ LayeredModel::~LayeredModel() {
     for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq})
         if (p) (void)hipFree(p);
     for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
+    if (attn_ws) (void)hipFree(attn_ws);
     for (void *p : {embed, head, (void *)x, (void *)proj, (void *)gu, (void *)tmp, (void *)ret_o, a1, a2, cat, xsel, (void *)in_dev}) if (p) (void)hipFree(p);
     if (in_host) (void)hipHostFree(in_host);
 }
@@ -84,6 +85,7 @@ int LayeredModel::init(nvr_model_runner &r) {
         RC(dmalloc(&w.canon1, (size_t)(W * taps * 4))); NVR_HIP_CHECK(hipMemset(w.canon1, 0, (size_t)(W * taps * 4)));
         RC(dmalloc(&w.canon2, (size_t)(W * taps * 4))); NVR_HIP_CHECK(hipMemset(w.canon2, 0, (size_t)(W * taps * 4)));
         if (L.mixer == LayeredSpec::ATTENTION) {
+            if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
             for (float **p : {&w.r1, &w.r2, &w.sink}) { RC(dmalloc(p, (size_t)L.heads * 4)); NVR_HIP_CHECK(hipMemset(*p, 0, (size_t)L.heads * 4)); }
         } else {
             std::vector<float> d(L.heads), f((size_t)std::max<int64_t>(L.rot_dims / 2, 1));
@@ -139,7 +141,10 @@ int LayeredModel::init(nvr_model_runner &r) {
     RC(dmalloc(&r.logits, (size_t)(logit_rows_cap * V * 4)));
 
     // step inputs: ids | row_seq | want | cu | start | slot | par | block tables
-    in_bytes = (size_t)(MT * 8 + MT * 4 * 2 + (r.max_seqs + 1) * 4 + r.max_seqs * 4 * 3 + r.max_seqs * r.max_blocks_per_seq * 4 + 256);
+    in_bytes = (size_t)(MT * 8 + MT * 4 * 2 + (r.max_seqs + 1) * 4 + r.max_seqs * 4 * 3 + r.max_seqs * r.max_blocks_per_seq * 4 + 256) +
+               attn_groups.size() * (size_t)((MT + r.max_seqs) * sizeof(kl::AttnTile) + 16);
+    attn_ws_bytes = kl::sink_attention_workspace_bytes(2 * r.num_cus);
+    NVR_HIP_CHECK(hipMalloc(&attn_ws, attn_ws_bytes));
     NVR_HIP_CHECK(hipHostMalloc((void **)&in_host, in_bytes, hipHostMallocDefault));
     NVR_HIP_CHECK(hipMalloc((void **)&in_dev, in_bytes));
 
@@ -258,7 +263,21 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
     auto carve = [&](size_t bytes) { size_t o = off; off += (bytes + 15) / 16 * 16; return o; };
     const size_t o_ids = carve((size_t)T * 8), o_rs = carve((size_t)T * 4), o_want = carve(std::max<size_t>(R, 1) * 4), o_cu = carve((nseq + 1) * 4), o_st = carve(nseq * 4),
                  o_sl = carve(nseq * 4), o_par = carve(nseq * 4), o_bt = carve(nseq * (size_t)MB * 4);
+    // query tiles of the matrix-core attention, one list per distinct group size g = H / G: 64 / g positions of one sequence each
+    std::vector<size_t> o_tiles(attn_groups.size()); std::vector<int32_t> n_tiles(attn_groups.size(), 0);
+    for (size_t gi = 0; gi < attn_groups.size(); ++gi) {
+        const int64_t pw = std::max<int64_t>(1, 64 / attn_groups[gi]);
+        size_t cnt = 0;
+        for (size_t i = 0; i < nseq; ++i) cnt += (seqs[i]->chunk_len + (size_t)pw - 1) / (size_t)pw;
+        o_tiles[gi] = carve(cnt * sizeof(kl::AttnTile)); n_tiles[gi] = (int32_t)cnt;
+    }
     if (off > in_bytes) return fail(NVR_ERR_INVARIANT, "execute_model: step inputs of %zu bytes exceed the arena", off);
+    for (size_t gi = 0; gi < attn_groups.size(); ++gi) {
+        const int64_t pw = std::max<int64_t>(1, 64 / attn_groups[gi]);
+        kl::AttnTile *tl = (kl::AttnTile *)(in_host + o_tiles[gi]);
+        for (size_t i = 0; i < nseq; ++i)
+            for (int64_t r0 = 0; r0 < (int64_t)seqs[i]->chunk_len; r0 += pw) *tl++ = kl::AttnTile{(int32_t)i, (int32_t)r0};
+    }
     int64_t *ids = (int64_t *)(in_host + o_ids); int32_t *rowseq = (int32_t *)(in_host + o_rs), *wnt = (int32_t *)(in_host + o_want), *cu = (int32_t *)(in_host + o_cu),
             *stt = (int32_t *)(in_host + o_st), *sl = (int32_t *)(in_host + o_sl), *par = (int32_t *)(in_host + o_par), *bt = (int32_t *)(in_host + o_bt);
     int64_t t = 0;
@@ -300,7 +319,15 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
             a.q = (const char *)proj + (size_t)(w.qcol * esz); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
             a.out = cat; a.ldo = w.kcat;
-            RC(kl::sink_attention(a, b, bf16, s));
+            if (kl::sink_attention_tiled_ok(a, bf16)) {
+                const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) - attn_groups.begin());
+                // decode-sized steps over long contexts: few tiles, many keys each — spread every tile's keys over several workgroups
+                const int64_t wgs = (int64_t)n_tiles[gi] * L.kv_heads;
+                int64_t nsplit = 1;
+                if (wgs < r.num_cus && max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / wgs, (max_ctx + 255) / 256, 16}));
+                RC(kl::sink_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + o_tiles[gi]), n_tiles[gi], (int)nsplit, attn_ws, attn_ws_bytes, s));
+            } else
+                RC(kl::sink_attention(a, b, bf16, s));
         } else {
             kl::RetentionArgs a{};
             a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.freq = w.freq; a.rot_dims = (int32_t)L.rot_dims;

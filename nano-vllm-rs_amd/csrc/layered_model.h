@@ -58,6 +58,8 @@ public:
     float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32
     void *proj = nullptr, *gu = nullptr, *tmp = nullptr, *a1 = nullptr, *a2 = nullptr, *cat = nullptr, *xsel = nullptr;   // operand type
     int64_t slots = 0; std::vector<int32_t> slot_par;
+    std::vector<int64_t> attn_groups;                       // distinct H / G of the attention layers: one list of query tiles per value and step
+    void *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // split-key partials of decode-sized steps
     // step inputs
     char *in_host = nullptr, *in_dev = nullptr; size_t in_bytes = 0;
     int64_t logit_rows_cap = 0;

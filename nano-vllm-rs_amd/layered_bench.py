@@ -1,0 +1,112 @@
+"""Prefill and decode throughput of a Rugudra-design model beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
+
+Random weights, layer shapes that resemble a real model's; both models go through the same engine (scheduler, block manager, runner step).
+Per size one JSON object: tokens/s of one prefill step over BATCH prompts of PROMPT tokens and of the decode steps that follow, for both."""
+import json
+import time
+
+import numpy as np
+
+SIZES = {
+    # width, ff, heads, kv_heads, head size, layers (alternating attention / retention for the layer-list model), vocab
+    "w1024": dict(width=1024, ff=3072, heads=16, kv_heads=8, dim=128, layers=4, vocab=32768),
+    "w2048": dict(width=2048, ff=6144, heads=16, kv_heads=8, dim=128, layers=4, vocab=32768),
+    "w4096": dict(width=4096, ff=12288, heads=32, kv_heads=8, dim=128, layers=2, vocab=32768),
+}
+
+
+def rugudra_config(s, loop=False):
+    layers = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            layers.append({"type": "attention", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5},
+                           "mlp": {"kind": "dense", "ff": s["ff"], "limit": 7.0}})
+        else:
+            h = s["heads"]
+            layers.append({"type": "retention", "mixer": {"heads": h, "dim": s["dim"], "vdim": s["dim"], "decay": [1.0 - 2.0 ** (-5 - 3 * j / max(1, h - 1)) for j in range(h)],
+                                                          "rot": {"dims": s["dim"], "base": 10000.0}},
+                           "mlp": {"kind": "dense", "ff": s["ff"], "limit": 7.0}})
+    cfg = {"architecture": "Rugudra", "vocab": s["vocab"], "width": s["width"], "residual_mult": 0.5, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+           "canon": {"taps": 4}, "layers": layers}
+    if loop:
+        cfg["loop"] = {"start": 0, "stop": len(layers), "times": 2}
+    return cfg
+
+
+def random_weights(cfg, seed=0):
+    """Tensors of a Rugudra configuration with values of a size that keeps activations in range (f32 arrays by name)."""
+    rng = np.random.default_rng(seed)
+    W, V, taps = cfg["width"], cfg["vocab"], cfg["canon"]["taps"]
+
+    def lin(o, i):
+        return (rng.standard_normal((o, i), dtype=np.float32) * (1.0 / np.sqrt(i))).astype(np.float32)
+    out = {"embed": rng.standard_normal((V, W), dtype=np.float32), "head": lin(V, W), "final.norm": np.float32(1.0)}
+    for i, L in enumerate(cfg["layers"]):
+        m, p = L["mixer"], "l%d." % i
+        H, D, Dv = m["heads"], m["dim"], m["vdim"]
+        G = m.get("kv_heads", H)
+        out[p + "norm1"] = np.float32(1.0 + 0.1 * rng.standard_normal())
+        out[p + "norm2"] = np.float32(1.0 + 0.1 * rng.standard_normal())
+        out[p + "canon1"] = (0.2 * rng.standard_normal((W, taps))).astype(np.float32)
+        out[p + "canon2"] = (0.2 * rng.standard_normal((W, taps))).astype(np.float32)
+        out[p + "mix.q"], out[p + "mix.k"], out[p + "mix.v"], out[p + "mix.o"] = lin(H * D, W), lin(G * D, W), lin(G * Dv, W), lin(W, H * Dv)
+        if L["type"] == "retention":
+            out[p + "mix.g"] = lin(H * Dv, W)
+        else:
+            out[p + "mix.r1"] = rng.uniform(0.1, 1.0, H).astype(np.float32)
+            out[p + "mix.r2"] = rng.uniform(0.05, 0.5, H).astype(np.float32)
+            out[p + "mix.sink"] = rng.standard_normal(H).astype(np.float32)
+        if L.get("mlp"):
+            F = L["mlp"]["ff"]
+            out[p + "mlp.gate"], out[p + "mlp.up"], out[p + "mlp.down"] = lin(F, W), lin(F, W), lin(W, F)
+    return out
+
+
+def _run(nvr, engine, vocab, batch, prompt, steps, warmup):
+    sp = nvr.SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
+    for i in range(batch):
+        engine.add_request(nvr.synthetic_tokens(prompt, 7, i, vocab).tolist(), sp)
+    nvr.synchronize()
+    t0 = time.perf_counter()
+    rec = engine.step()
+    nvr.synchronize()
+    t_prefill = time.perf_counter() - t0
+    assert rec["is_prefill"] and rec["num_seqs"] == batch, rec
+    for _ in range(warmup):
+        engine.step()
+    nvr.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    nvr.synchronize()
+    t_decode = (time.perf_counter() - t0) / steps
+    return dict(prefill_tokens_per_s=round(batch * prompt / t_prefill), prefill_ms=round(t_prefill * 1e3, 2),
+                decode_tokens_per_s=round(batch / t_decode), decode_ms_per_step=round(t_decode * 1e3, 3))
+
+
+def compare(nvr, sizes=("w1024", "w2048"), batch=16, prompt=1024, steps=32, warmup=4, dtype="bfloat16", which=("rugudra", "qwen3")):
+    out = []
+    bs = 256
+    for name in sizes:
+        s = SIZES[name]
+        ecfg = dict(max_num_seqs=batch, max_num_batched_tokens=batch * prompt, max_model_len=prompt + steps + warmup + 8, kvcache_block_size=bs,
+                    num_kvcache_blocks=batch * ((prompt + steps + warmup + 8 + bs - 1) // bs + 1), dtype=dtype)
+        line = {"size": name, "shape": s, "batch": batch, "prompt_len": prompt, "decode_steps": steps, "dtype": dtype}
+        if "rugudra" in which:
+            cfg = rugudra_config(s)
+            eng = nvr.LLMEngine(nvr.Config(**ecfg), nvr.ModelSpec(cfg))
+            for k, v in random_weights(cfg).items():
+                eng.model_runner.load_tensor(k, np.asarray(v))
+            _run(nvr, eng, s["vocab"], 2, 64, 2, 1)                       # first launches
+            line["rugudra"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
+            del eng
+        if "qwen3" in which:
+            m = nvr.ModelConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
+                                num_key_value_heads=s["kv_heads"], head_dim=s["dim"], max_position_embeddings=8192, tie_word_embeddings=0)
+            eng = nvr.LLMEngine(nvr.Config(**ecfg), m)
+            _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
+            line["qwen3"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
+            del eng
+        out.append(line)
+        print(json.dumps(line), flush=True)
+    return out
