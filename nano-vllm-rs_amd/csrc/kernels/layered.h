@@ -35,7 +35,7 @@ int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, f
 // rows of K ([G][D]) and V ([G][Dv]) out of the projection rows (operand type) (row stride ld; column offsets kcol / vcol) into the paged caches
 // [blocks][block_size][G][D] / [..][Dv] at the rows' positions
 int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
-             hipStream_t s);
+             bool v_grouped, hipStream_t s);   // v_grouped: the value page layout of the tiled attention, [block][block_size / 8][G][Dv][8 keys]
 
 // Causal softmax attention through the block tables: query row t at position i sees keys j <= i of its sequence;
 // score = q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)); the denominator also holds exp(sink[h]) (no key, no value).  r1 / r2 / sink may be null (plain
@@ -46,13 +46,16 @@ struct SinkAttnArgs {
     const float *r1, *r2, *sink;
     int32_t H, G, D, Dv; float scale;
     void *out; int64_t ldo;
+    const float *pen; int32_t pen_n;         // tiled form: penalty_table of this layer ([H][pen_n]; null: no penalty)
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
 // rows row0 .. row0 + 64 / (H / G) - 1 of sequence seq's chunk, for all H / G query heads of a key/value head.  nsplit > 1 spreads a tile's keys over that many
 // workgroups (decode-sized steps over long contexts) and merges their partials; workspace: sink_attention_workspace_bytes(ntiles * G * nsplit).
 struct AttnTile { int32_t seq, row0; };
-bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16);
+bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size);   // (pages of a multiple of 8 tokens)
+// tab[h][d] = r1[h] * ln(1 + r2[h] * d) * log2(e) for d < n: the penalty the tiled form subtracts in the base-2 domain
+int penalty_table(const float *r1, const float *r2, int64_t H, int64_t n, float *tab, hipStream_t s);
 size_t sink_attention_workspace_bytes(int max_workgroups);
 int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s);
 

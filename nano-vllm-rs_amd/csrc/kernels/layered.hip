@@ -120,14 +120,17 @@ __global__ __launch_bounds__(256) void norm_canon_kernel(const float *__restrict
 // ------------------------------------------------------------------------------------------------ K / V rows into the paged caches
 template <class CT>
 __global__ __launch_bounds__(256) void kv_store_kernel(const CT *__restrict__ proj, int64_t ld, int64_t kcol, int64_t vcol, Batch b, int G, int D, int Dv,
-                                                       CT *__restrict__ kc, CT *__restrict__ vc) {
+                                                       CT *__restrict__ kc, CT *__restrict__ vc, int grouped) {
     const int t = blockIdx.x, sq = b.row_seq[t];
     const int p = b.start[sq] + (t - b.cu[sq]);
     const int blk = b.block_tables[(int64_t)sq * b.max_blocks + p / b.block_size];
     const int64_t row = (int64_t)blk * b.block_size + p % b.block_size;
     const CT *pr = proj + (int64_t)t * ld;
     for (int c = threadIdx.x; c < G * D; c += 256) kc[row * G * D + c] = pr[kcol + c];
-    for (int c = threadIdx.x; c < G * Dv; c += 256) vc[row * G * Dv + c] = pr[vcol + c];
+    if (!grouped) { for (int c = threadIdx.x; c < G * Dv; c += 256) vc[row * G * Dv + c] = pr[vcol + c]; return; }
+    const int jj = p % b.block_size;                    // value pages in groups of 8 keys per column: [block][block_size / 8][G][Dv][8]
+    const int64_t grp = ((int64_t)blk * (b.block_size >> 3) + (jj >> 3)) * G * Dv;
+    for (int c = threadIdx.x; c < G * Dv; c += 256) vc[(grp + c) * 8 + (jj & 7)] = pr[vcol + c];
 }
 
 // ------------------------------------------------------------------------------------------------ attention with distance penalty and sink
@@ -186,19 +189,29 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
 // Matrix-core form (bf16 operands; D and Dv multiples of 32 / 16 up to the size class C).  A workgroup owns one tile — up to 64 / g consecutive
 // positions of one sequence times the g = H / G query heads of one key/value head, 16 rows per wave — and walks the keys in tiles of 64 through LDS:
 // S = Q K^T on v_mfma_f32_16x16x32_bf16, penalty / mask / online softmax in f32 on the accumulator layout (lane: key column, four rows), P rounded
-// to bf16 through LDS into the A layout, O += P V with V held transposed in LDS.  The sink starts the running maximum and counts 1 in the running
-// sum.  nsplit > 1: workgroup z takes every nsplit-th share of the keys and leaves (o, m, l) partials for sink_attn_merge_kernel.
+// to bf16 through LDS into the A layout, O += P V.  The value pages are stored in groups of 8 keys per column ([.][G][Dv][8]), so that a B fragment
+// of P V (8 consecutive keys of one column) is one 16-byte read.  The distance penalty comes from a table per head (penalty_table_kernel), everything
+// in the base-2 domain (v_exp_f32 is 2^x).  The next tile's keys and values are requested before the current tile's arithmetic and land in LDS after
+// it.  The sink starts the running maximum and counts 1 in the running sum.  nsplit > 1: workgroup z takes every nsplit-th tile of keys and leaves
+// (o, m, l) partials for sink_attn_merge_kernel.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr float kLog2e = 1.4426950408889634f;
+
+__global__ __launch_bounds__(256) void penalty_table_kernel(const float *__restrict__ r1, const float *__restrict__ r2, int H, int n, float *__restrict__ tab) {
+    const int d = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y;
+    if (d < n) tab[(int64_t)h * n + d] = r1[h] * log1pf(r2[h] * (float)d) * kLog2e;
+}
 
 template <int C>
 __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, float *__restrict__ part_o,
                                                              float *__restrict__ part_ml) {
-    constexpr int KT = 64, KS = C + 8, VS = KT + 8;
+    constexpr int KT = 64, KS = C + 8, VS = KT + 8, VG = C + 1, NCH = C / 32;   // NCH: 16-byte pieces of a K (or V) tile per thread
     extern __shared__ char smem[];
     bf16_t *Ks = (bf16_t *)smem;                        // [KT][KS] keys x dims
-    bf16_t *Vt = Ks + KT * KS;                          // [C][VS] value columns x keys
-    bf16_t *Ps = Vt + C * VS;                           // [4][16][VS] one wave's weights
+    bf16_t *Vg = Ks + KT * KS;                          // [8 key groups][VG columns][8 keys]
+    bf16_t *Ps = Vg + 8 * VG * 8;                       // [4][16][VS] one wave's weights
+    float *pen = (float *)(Ps + 64 * VS);               // [g][128] penalties of the distances this key tile can have
     const int tile = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
     const int sq = tiles[tile].seq, lr0 = tiles[tile].row0;
     const int c0 = b.cu[sq], n = b.cu[sq + 1] - c0, st = b.start[sq];
@@ -209,6 +222,8 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
     const bool wave_on = wave * 16 < npos * g;
     const bf16_t *kc = (const bf16_t *)a.kc, *vc = (const bf16_t *)a.vc;
     const int32_t *bt = b.block_tables + (int64_t)sq * b.max_blocks;
+    const int bs = b.block_size, bs8 = bs >> 3;
+    const float scale2 = a.scale * kLog2e;
 
     bf16x8 qf[C / 32];
     {
@@ -217,47 +232,57 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
 #pragma unroll
         for (int ks = 0; ks < C / 32; ++ks) if (ks < d32) qf[ks] = *reinterpret_cast<const bf16x8 *>(q + ks * 32);
     }
-    int pos[4]; float r1[4], r2[4], m[4], l[4];
+    int pos[4], hgi[4]; float m[4], l[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = wave * 16 + lq * 4 + i, h = kvh * g + r % g;
-        pos[i] = st + lr0 + r / g;
-        r1[i] = a.r1 ? a.r1[h] : 0.f; r2[i] = a.r2 ? a.r2[h] : 0.f;
+        pos[i] = st + lr0 + r / g; hgi[i] = r % g;
         const bool sink_here = a.sink && z == 0;
-        m[i] = sink_here ? a.sink[h] : -INFINITY;
+        m[i] = sink_here ? a.sink[h] * kLog2e : -INFINITY;
         l[i] = (sink_here && lm == 0) ? 1.f : 0.f;
     }
     f32x4 acc[C / 16];
 #pragma unroll
     for (int t = 0; t < C / 16; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nkeys = st + lr0 + npos;                  // keys the tile's last position sees
+    const int p0 = st + lr0;                            // first position of the tile
+    const int nkeys = p0 + npos;                        // keys the tile's last position sees
     const int ntl = (nkeys + KT - 1) / KT;
+    const int kch = D >> 3;
+    uint4 kreg[NCH], vreg[NCH];
+    auto request = [&](int k0) {                        // pieces of the key tile at k0 -> registers
+#pragma unroll
+        for (int x = 0; x < NCH; ++x) {
+            const int idx = threadIdx.x + x * 256;
+            kreg[x] = uint4{0, 0, 0, 0}; vreg[x] = uint4{0, 0, 0, 0};
+            if (idx < KT * kch) {
+                const int key = idx / kch, ch = idx - key * kch, j = k0 + key;
+                if (j < nkeys) kreg[x] = *reinterpret_cast<const uint4 *>(kc + (((int64_t)bt[j / bs] * bs + j % bs) * a.G + kvh) * D + ch * 8);
+            }
+            if (idx < 8 * Dv) {
+                const int kg = idx / Dv, c = idx - kg * Dv, j = k0 + kg * 8;
+                if (j < nkeys) vreg[x] = *reinterpret_cast<const uint4 *>(vc + ((((int64_t)bt[j / bs] * bs8 + ((j % bs) >> 3)) * a.G + kvh) * Dv + c) * 8);
+            }
+        }
+    };
+    if (z < ntl) request(z * KT);
     for (int kt = z; kt < ntl; kt += nsplit) {
         const int k0 = kt * KT;
+        const int dmin = max(p0 - (k0 + KT - 1), 0);    // smallest distance a visible key of this tile can have
         __syncthreads();
-        const int kch = D >> 3, vch = Dv >> 3;
-        for (int idx = threadIdx.x; idx < KT * kch; idx += 256) {
-            const int key = idx / kch, ch = idx - key * kch, j = k0 + key;
-            uint4 v = uint4{0, 0, 0, 0};
-            if (j < nkeys) {
-                const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
-                v = *reinterpret_cast<const uint4 *>(kc + (row * a.G + kvh) * D + ch * 8);
-            }
-            *reinterpret_cast<uint4 *>(Ks + key * KS + ch * 8) = v;
-        }
-        for (int idx = threadIdx.x; idx < KT * vch; idx += 256) {
-            const int ch = idx / KT, key = idx - ch * KT, j = k0 + key;      // (consecutive threads: consecutive keys of one column block)
-            uint4 v = uint4{0, 0, 0, 0};
-            if (j < nkeys) {
-                const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
-                v = *reinterpret_cast<const uint4 *>(vc + (row * a.G + kvh) * Dv + ch * 8);
-            }
-            const bf16_t *e = reinterpret_cast<const bf16_t *>(&v);
 #pragma unroll
-            for (int x = 0; x < 8; ++x) Vt[(ch * 8 + x) * VS + key] = e[x];
+        for (int x = 0; x < NCH; ++x) {
+            const int idx = threadIdx.x + x * 256;
+            if (idx < KT * kch) { const int key = idx / kch, ch = idx - key * kch; *reinterpret_cast<uint4 *>(Ks + key * KS + ch * 8) = kreg[x]; }
+            if (idx < 8 * Dv) { const int kg = idx / Dv, c = idx - kg * Dv; *reinterpret_cast<uint4 *>(Vg + (kg * VG + c) * 8) = vreg[x]; }
         }
+        if (a.pen)
+            for (int idx = threadIdx.x; idx < g * 128; idx += 256) {
+                const int hg = idx >> 7, d = dmin + (idx & 127);
+                pen[idx] = d < a.pen_n ? a.pen[(int64_t)(kvh * g + hg) * a.pen_n + d] : 0.f;
+            }
         __syncthreads();
+        if (kt + nsplit < ntl) request((kt + nsplit) * KT);
         if (wave_on) {
             f32x4 s[4];
 #pragma unroll
@@ -276,9 +301,10 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
                 const int j = k0 + nt * 16 + lm;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float v = s[nt][i] * a.scale;
-                    if (a.r1) v -= r1[i] * __logf(1.0f + r2[i] * (float)(pos[i] - j));
-                    v = (j > pos[i]) ? -INFINITY : v;
+                    const int dist = pos[i] - j;
+                    float v = s[nt][i] * scale2;
+                    if (a.pen) v -= pen[(hgi[i] << 7) + min(max(dist - dmin, 0), 127)];
+                    v = dist < 0 ? -INFINITY : v;
                     s[nt][i] = v;
                     mx[i] = fmaxf(mx[i], v);
                 }
@@ -288,29 +314,29 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
 #pragma unroll
                 for (int o = 1; o < 16; o <<= 1) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], o, 64));
                 const float mn = fmaxf(m[i], mx[i]);
-                const float alpha = (m[i] == -INFINITY) ? 0.f : __expf(m[i] - mn);
+                const float alpha = (m[i] == -INFINITY) ? 0.f : exp2f(m[i] - mn);
+                const float ms = (mn == -INFINITY) ? 0.f : mn;
                 m[i] = mn;
                 float rs = 0.f;
 #pragma unroll
                 for (int nt = 0; nt < 4; ++nt) {
-                    const float p = (s[nt][i] == -INFINITY) ? 0.f : __expf(s[nt][i] - mn);
+                    const float p = exp2f(s[nt][i] - ms);                // (a masked key: 2^-inf = 0)
                     rs += p;
-                    st_f(Ps, (wave * 16 + lq * 4 + i) * VS + nt * 16 + lm, p);
+                    const __bf16 pb = (__bf16)p;
+                    Ps[(wave * 16 + lq * 4 + i) * VS + nt * 16 + lm] = __builtin_bit_cast(bf16_t, pb);
                 }
                 l[i] = l[i] * alpha + rs;
 #pragma unroll
                 for (int t = 0; t < C / 16; ++t) acc[t][i] *= alpha;
             }
-        }
-        __syncthreads();
-        if (wave_on) {
+            __builtin_amdgcn_wave_barrier();                // (the weights are read back by this wave only: LDS serves a wave's requests in order)
 #pragma unroll
             for (int k2 = 0; k2 < KT / 32; ++k2) {
                 const bf16x8 pf = *reinterpret_cast<const bf16x8 *>(Ps + (wave * 16 + lm) * VS + k2 * 32 + lq * 8);
 #pragma unroll
                 for (int t = 0; t < C / 16; ++t)
                     if (t < dv16) {
-                        const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(Vt + (t * 16 + lm) * VS + k2 * 32 + lq * 8);
+                        const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(Vg + ((k2 * 4 + lq) * VG + t * 16 + lm) * 8);
                         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc[t], 0, 0, 0);
                     }
             }
@@ -337,7 +363,7 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
     }
 }
 
-// one wave per (tile, key/value head, row): out = sum_z o_z e^(m_z - m) / sum_z l_z e^(m_z - m)
+// one wave per (tile, key/value head, row): out = sum_z o_z 2^(m_z - m) / sum_z l_z 2^(m_z - m)
 __global__ __launch_bounds__(64) void sink_attn_merge_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, const float *__restrict__ part_o,
                                                              const float *__restrict__ part_ml) {
     const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
@@ -350,11 +376,11 @@ __global__ __launch_bounds__(64) void sink_attn_merge_kernel(SinkAttnArgs a, Bat
     float m = -INFINITY;
     for (int z = 0; z < nsplit; ++z) m = fmaxf(m, part_ml[((base + z) * 64 + r) * 2]);
     float l = 0.f;
-    for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) l += part_ml[((base + z) * 64 + r) * 2 + 1] * __expf(mz - m); }
+    for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) l += part_ml[((base + z) * 64 + r) * 2 + 1] * exp2f(mz - m); }
     bf16_t *o = (bf16_t *)a.out + (int64_t)(c0 + lr0 + pi) * a.ldo + (int64_t)(kvh * g + hg) * a.Dv;
     for (int c = threadIdx.x; c < a.Dv; c += 64) {
         float acc = 0.f;
-        for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) acc += part_o[((base + z) * 64 + r) * a.Dv + c] * __expf(mz - m); }
+        for (int z = 0; z < nsplit; ++z) { const float mz = part_ml[((base + z) * 64 + r) * 2]; if (mz != -INFINITY) acc += part_o[((base + z) * 64 + r) * a.Dv + c] * exp2f(mz - m); }
         st_f(o, c, acc / l);
     }
 }
@@ -508,22 +534,23 @@ int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, f
 }
 
 int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Batch &b, int64_t G, int64_t D, int64_t Dv, void *kc, void *vc, bool bf16,
-             hipStream_t s) {
+             bool v_grouped, hipStream_t s) {
+    if (v_grouped && b.block_size % 8) return nvr::fail(NVR_ERR_INVALID_ARG, "kv_store: grouped value pages need a block size that is a multiple of 8");
     if (b.T == 0) return 0;
-    if (bf16) kv_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (bf16_t *)kc, (bf16_t *)vc);
-    else kv_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (float *)kc, (float *)vc);
+    if (bf16) kv_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const bf16_t *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (bf16_t *)kc, (bf16_t *)vc, (int)v_grouped);
+    else kv_store_kernel<float><<<dim3((unsigned)b.T), dim3(256), 0, s>>>((const float *)proj, ld, kcol, vcol, b, (int)G, (int)D, (int)Dv, (float *)kc, (float *)vc, (int)v_grouped);
     return launched("kv_store");
 }
 
-bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16) {
-    return bf16 && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
+bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size) {
+    return bf16 && block_size % 8 == 0 && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
            ((uintptr_t)a.q % 16) == 0 && ((uintptr_t)a.kc % 16) == 0 && ((uintptr_t)a.vc % 16) == 0;
 }
 size_t sink_attention_workspace_bytes(int max_workgroups) { return (size_t)max_workgroups * 64 * (256 + 2) * sizeof(float); }
 
 int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s) {
     if (ntiles == 0) return 0;
-    if (!sink_attention_tiled_ok(a, true)) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention_tiled: shape outside the matrix-core kernel");
+    if (!sink_attention_tiled_ok(a, true, b.block_size)) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention_tiled: shape outside the matrix-core kernel");
     if (nsplit < 1) nsplit = 1;
     float *po = nullptr, *pml = nullptr;
     if (nsplit > 1) {
@@ -532,7 +559,7 @@ int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *
         po = (float *)workspace; pml = po + rows * a.Dv;
     }
     const int C = std::max(a.D, a.Dv) <= 64 ? 64 : std::max(a.D, a.Dv) <= 128 ? 128 : 256;
-    const size_t lds = ((size_t)64 * (C + 8) + (size_t)C * 72 + (size_t)64 * 72) * 2;
+    const size_t lds = ((size_t)64 * (C + 8) + (size_t)8 * (C + 1) * 8 + (size_t)64 * 72) * 2 + (size_t)(a.H / a.G) * 128 * 4;
     const dim3 grid((unsigned)ntiles, (unsigned)a.G, (unsigned)nsplit);
     if (C == 64) sink_attn_mfma_kernel<64><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
     else if (C == 128) sink_attn_mfma_kernel<128><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
@@ -543,6 +570,12 @@ int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *
         return launched("sink_attention merge");
     }
     return 0;
+}
+
+int penalty_table(const float *r1, const float *r2, int64_t H, int64_t n, float *tab, hipStream_t s) {
+    if (H * n == 0) return 0;
+    penalty_table_kernel<<<dim3((unsigned)((n + 255) / 256), (unsigned)H), dim3(256), 0, s>>>(r1, r2, (int)H, (int)n, tab);
+    return launched("penalty_table");
 }
 
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s) {

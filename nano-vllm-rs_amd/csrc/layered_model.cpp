@@ -39,7 +39,7 @@ inline float src_at(int dtype, const void *src, size_t i) {
 }  // namespace
 
 LayeredModel::~LayeredModel() {
-    for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq})
+    for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq, (void *)w.pen})
         if (p) (void)hipFree(p);
     for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
     if (attn_ws) (void)hipFree(attn_ws);
@@ -210,8 +210,8 @@ int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtyp
     if (rest == "mix.o") return is2(W, hv) ? put(r, w.out, w.kcat, W, hv, dtype, data, true) : bad();
     if (L.mixer == LayeredSpec::RETENTION && rest == "mix.g") return is2(hv, W) ? put(r, rows_at(w.mix, w.gcol, W), W, hv, W, dtype, data, true) : bad();
     if (L.mixer == LayeredSpec::ATTENTION) {
-        if (rest == "mix.r1") return vec(w.r1, L.heads);
-        if (rest == "mix.r2") return vec(w.r2, L.heads);
+        if (rest == "mix.r1") { w.pen_dirty = true; return vec(w.r1, L.heads); }
+        if (rest == "mix.r2") { w.pen_dirty = true; return vec(w.r2, L.heads); }
         if (rest == "mix.sink") return vec(w.sink, L.heads);
     }
     if (L.has_mlp) {
@@ -314,12 +314,20 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
         RC(kl::norm_canon(x, b, W, eps, (int)spec.taps, w.g1, w.canon1, a1, w.g2, w.canon2, L.has_mlp ? a2 : nullptr, bf16, st.hist, slots, s));
         RC(gemm(r, a1, W, w.mix, T, W, w.nmix, proj));
         if (L.mixer == LayeredSpec::ATTENTION) {
-            RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, s));
             kl::SinkAttnArgs a{};
             a.q = (const char *)proj + (size_t)(w.qcol * esz); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
             a.out = cat; a.ldo = w.kcat;
-            if (kl::sink_attention_tiled_ok(a, bf16)) {
+            const bool tiled = kl::sink_attention_tiled_ok(a, bf16, (int)r.block_size);   // (a property of the layer's shape: the same answer every step)
+            RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, tiled, s));
+            if (tiled) {
+                LayerW &wm = lw[li];
+                if (!wm.pen || wm.pen_dirty) {                                      // the penalties by distance, once per set of r1 / r2
+                    if (!wm.pen) RC(dmalloc(&wm.pen, (size_t)(L.heads * r.max_pos * 4)));
+                    RC(kl::penalty_table(w.r1, w.r2, L.heads, r.max_pos, wm.pen, s));
+                    wm.pen_dirty = false;
+                }
+                a.pen = wm.pen; a.pen_n = (int32_t)r.max_pos;
                 const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) - attn_groups.begin());
                 // decode-sized steps over long contexts: few tiles, many keys each — spread every tile's keys over several workgroups
                 const int64_t wgs = (int64_t)n_tiles[gi] * L.kv_heads;

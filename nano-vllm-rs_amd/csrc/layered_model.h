@@ -47,6 +47,7 @@ public:
         float *canon1 = nullptr, *canon2 = nullptr;         // [W][taps]
         float *r1 = nullptr, *r2 = nullptr, *sink = nullptr, *decay = nullptr, *freq = nullptr;
         float g1 = 1.f, g2 = 1.f;
+        float *pen = nullptr; bool pen_dirty = true;        // attention on the matrix cores: r1 * ln(1 + r2 * d) by head and distance
         int64_t nmix = 0, kcat = 0, mixcols = 0;            // rows of mix, columns of out, of which the mixer's
         int64_t qcol = 0, kcol = 0, vcol = 0, gcol = 0;
     };
