@@ -60,11 +60,11 @@ size_t sink_attention_workspace_bytes(int max_workgroups);
 int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s);
 
 // Retention over the rows of a step: per head S <- decay[h] * S + k v^T, o = S^T q, with q and k rotated (first rot_dims coordinates, pairs (i, i + rot_dims/2),
-// angle = position * freq[i]) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: rows of the operand type (stride ld) holding
+// angle = position * freq[i], cosines and sines from a table) and k scaled by kscale after the rotation.  state: [slots][H][D][Dv] f32, zero at position 0.  proj: rows of the operand type (stride ld) holding
 // q at column qcol ([H][D]), k at kcol, v at vcol ([H][Dv]).  o: f32 [T][H*Dv].
 struct RetentionArgs {
     const void *proj; int64_t ld, qcol, kcol, vcol;
-    const float *decay, *freq; int32_t rot_dims; float kscale;
+    const float *decay, *cos_t, *sin_t; int32_t rot_dims; float kscale;   // cos_t / sin_t: [positions][rot_dims / 2] of angle = position * freq[i]
     int32_t H, D, Dv;
     float *state; float *o;
 };

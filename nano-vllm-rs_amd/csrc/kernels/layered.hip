@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void penalty_table_kernel(const float *__restr
 }
 
 template <int C>
-__global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, float *__restrict__ part_o,
+__global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, Batch b, const AttnTile *__restrict__ tiles, int nsplit, float *__restrict__ part_o,
                                                              float *__restrict__ part_ml) {
     constexpr int KT = 64, KS = C + 8, VS = KT + 8, VG = C + 1, NCH = C / 32;   // NCH: 16-byte pieces of a K (or V) tile per thread
     extern __shared__ char smem[];
@@ -250,19 +250,18 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
     const int ntl = (nkeys + KT - 1) / KT;
     const int kch = D >> 3;
     uint4 kreg[NCH], vreg[NCH];
+    // a thread's pieces: key skey, 16-byte pieces sch, sch + 4, ... of its row; key group vkg, columns vcl, vcl + 32, ... (one block-table lookup each per tile)
+    const int skey = threadIdx.x >> 2, sch = threadIdx.x & 3, vkg = threadIdx.x >> 5, vcl = threadIdx.x & 31;
     auto request = [&](int k0) {                        // pieces of the key tile at k0 -> registers
+        const int jk = k0 + skey, jv = k0 + vkg * 8;
+        const int bk = jk < nkeys ? jk / bs : 0, bv = jv < nkeys ? jv / bs : 0;
+        const bf16_t *kr = kc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * D;
+        const bf16_t *vr = vc + (((int64_t)bt[bv] * bs8 + ((jv - bv * bs) >> 3)) * a.G + kvh) * Dv * 8;
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
-            const int idx = threadIdx.x + x * 256;
             kreg[x] = uint4{0, 0, 0, 0}; vreg[x] = uint4{0, 0, 0, 0};
-            if (idx < KT * kch) {
-                const int key = idx / kch, ch = idx - key * kch, j = k0 + key;
-                if (j < nkeys) kreg[x] = *reinterpret_cast<const uint4 *>(kc + (((int64_t)bt[j / bs] * bs + j % bs) * a.G + kvh) * D + ch * 8);
-            }
-            if (idx < 8 * Dv) {
-                const int kg = idx / Dv, c = idx - kg * Dv, j = k0 + kg * 8;
-                if (j < nkeys) vreg[x] = *reinterpret_cast<const uint4 *>(vc + ((((int64_t)bt[j / bs] * bs8 + ((j % bs) >> 3)) * a.G + kvh) * Dv + c) * 8);
-            }
+            if (jk < nkeys && sch + 4 * x < kch) kreg[x] = *reinterpret_cast<const uint4 *>(kr + (sch + 4 * x) * 8);
+            if (jv < nkeys && vcl + 32 * x < Dv) vreg[x] = *reinterpret_cast<const uint4 *>(vr + (vcl + 32 * x) * 8);
         }
     };
     if (z < ntl) request(z * KT);
@@ -272,9 +271,8 @@ __global__ __launch_bounds__(256) void sink_attn_mfma_kernel(SinkAttnArgs a, Bat
         __syncthreads();
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
-            const int idx = threadIdx.x + x * 256;
-            if (idx < KT * kch) { const int key = idx / kch, ch = idx - key * kch; *reinterpret_cast<uint4 *>(Ks + key * KS + ch * 8) = kreg[x]; }
-            if (idx < 8 * Dv) { const int kg = idx / Dv, c = idx - kg * Dv; *reinterpret_cast<uint4 *>(Vg + (kg * VG + c) * 8) = vreg[x]; }
+            if (sch + 4 * x < kch) *reinterpret_cast<uint4 *>(Ks + skey * KS + (sch + 4 * x) * 8) = kreg[x];
+            if (vcl + 32 * x < Dv) *reinterpret_cast<uint4 *>(Vg + (vkg * VG + vcl + 32 * x) * 8) = vreg[x];
         }
         if (a.pen)
             for (int idx = threadIdx.x; idx < g * 128; idx += 256) {
@@ -408,8 +406,8 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
             float qv = ld_f(q, d), kv = ld_f(k, d);
             if (d < a.rot_dims) {
                 const int fi = d < half ? d : d - half;
-                const float ang = (float)(st + i) * a.freq[fi];
-                float sn, cs; sincosf(ang, &sn, &cs);
+                const int64_t p = st + i;
+                const float cs = a.cos_t[p * half + fi], sn = a.sin_t[p * half + fi];
                 if (d < half) { qv = qv * cs - ld_f(q, d + half) * sn; kv = kv * cs - ld_f(k, d + half) * sn; }
                 else { qv = qv * cs + ld_f(q, d - half) * sn; kv = kv * cs + ld_f(k, d - half) * sn; }
             }
@@ -438,18 +436,96 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
         for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; if (d < D) S[(int64_t)d * Dv + c] = s[r]; }
 }
 
+// The same recurrence, 16 tokens per barrier round (key size up to 256): a round brings the rotated q, scaled rotated k and v of its tokens into LDS (cosines
+// and sines from the position table), every thread then walks the tokens with its rows of the state in registers and leaves its partial outputs in LDS; one
+// barrier later they are summed over the 8 row groups.  Token order and arithmetic per token are those of the token-by-token kernel: the result does not depend
+// on where a prompt is cut.  Thread (c, part) owns rows part * RMAX .. part * RMAX + RMAX - 1 of column c.
+template <int RMAX, class PT>
+__global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, Batch b) {
+    constexpr int TB = 16;
+    extern __shared__ float rsm[];
+    const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
+    float *qs = rsm, *ks = qs + TB * D, *vs = ks + TB * D, *partial = vs + TB * 32;      // [TB][D], [TB][D], [TB][32], [TB][8][32]
+    const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
+    const int cl = threadIdx.x & 31, c = cb + cl, part = threadIdx.x >> 5;
+    const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
+    const float dec = a.decay[h];
+    float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
+    const bool live = c < Dv;
+    float s[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; s[r] = (st > 0 && live && d < D) ? S[(int64_t)d * Dv + c] : 0.f; }
+    for (int i0 = 0; i0 < n; i0 += TB) {
+        const int nb = min(TB, n - i0);
+        __syncthreads();
+        const int dsh = (D & (D - 1)) == 0 ? 31 - __clz(D) : -1;
+        for (int idx = threadIdx.x; idx < nb * D; idx += 256) {
+            const int i = dsh >= 0 ? idx >> dsh : idx / D, d = idx - i * D;
+            const PT *pr = (const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
+            const PT *q = pr + a.qcol + (int64_t)h * D, *k = pr + a.kcol + (int64_t)h * D;
+            float qv = ld_f(q, d), kv = ld_f(k, d);
+            if (d < a.rot_dims) {
+                const int fi = d < half ? d : d - half;
+                const int64_t p = st + i0 + i;
+                const float cs = a.cos_t[p * half + fi], sn = a.sin_t[p * half + fi];
+                if (d < half) { qv = qv * cs - ld_f(q, d + half) * sn; kv = kv * cs - ld_f(k, d + half) * sn; }
+                else { qv = qv * cs + ld_f(q, d - half) * sn; kv = kv * cs + ld_f(k, d - half) * sn; }
+            }
+            qs[idx] = qv; ks[idx] = kv * a.kscale;
+        }
+        for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
+            const int i = idx >> 5, cc = cb + (idx & 31);
+            vs[idx] = cc < Dv ? ld_f((const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld, a.vcol + (int64_t)h * Dv + cc) : 0.f;
+        }
+        __syncthreads();
+        for (int i = 0; i < nb; ++i) {
+            const float v = vs[i * 32 + cl];
+            const float *kr = ks + i * D + part * RMAX, *qr = qs + i * D + part * RMAX;
+            float o = 0.f;
+            if (D == 8 * RMAX) {
+                float kk[RMAX], qq[RMAX];
+#pragma unroll
+                for (int r = 0; r < RMAX; r += 4) {
+                    *reinterpret_cast<float4 *>(kk + r) = *reinterpret_cast<const float4 *>(kr + r);
+                    *reinterpret_cast<float4 *>(qq + r) = *reinterpret_cast<const float4 *>(qr + r);
+                }
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r) { s[r] = dec * s[r] + kk[r] * v; o += s[r] * qq[r]; }
+            } else {
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r)
+                    if (part * RMAX + r < D) { s[r] = dec * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+            }
+            partial[(i * 8 + part) * 32 + cl] = o;
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
+            const int i = idx >> 5, cc = cb + (idx & 31);
+            float tot = 0.f;
+#pragma unroll
+            for (int p2 = 0; p2 < 8; ++p2) tot += partial[(i * 8 + p2) * 32 + (idx & 31)];
+            if (cc < Dv) a.o[(int64_t)(r0 + i0 + i) * a.H * Dv + (int64_t)h * Dv + cc] = tot;
+        }
+    }
+    if (live)
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) { const int d = part * RMAX + r; if (d < D) S[(int64_t)d * Dv + c] = s[r]; }
+}
+
 template <class OT>
-__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float *__restrict__ o, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
-                                                            float eps, OT *__restrict__ out, int64_t ldo) {
-    const int64_t t = blockIdx.x; const int h = blockIdx.y;
-    const float *orow = o + (t * H + h) * Dv;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < Dv; c += 64) { const float v = orow[c]; ss += v * v; }
-    ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
-    for (int c = threadIdx.x; c < Dv; c += 64) {
-        const float g = ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c);
-        st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (g / (1.0f + expf(-g))));
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float *__restrict__ o, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
+                                                             float eps, OT *__restrict__ out, int64_t ldo) {
+    const int64_t t = blockIdx.x; const int lane = threadIdx.x & 63;
+    for (int h = threadIdx.x >> 6; h < H; h += 4) {              // a wave per head
+        const float *orow = o + (t * H + h) * Dv;
+        float ss = 0.f;
+        for (int c = lane; c < Dv; c += 64) { const float v = orow[c]; ss += v * v; }
+        ss = wave_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
+        for (int c = lane; c < Dv; c += 64) {
+            const float g = ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c);
+            st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (g / (1.0f + expf(-g))));
+        }
     }
 }
 
@@ -461,6 +537,23 @@ __global__ __launch_bounds__(256) void clamped_glu_kernel(const OT *__restrict__
     const float g = fminf(ld_f(gu, t * 2 * F + c), limit);
     const float u = fminf(fmaxf(ld_f(gu, t * 2 * F + F + c), -limit), limit);
     st_f(out, t * ldo + c, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+}
+
+template <class YT>
+// the same, 8 bf16 elements (16 bytes) per thread: F and ldo multiples of 8
+__global__ __launch_bounds__(256) void clamped_glu8_kernel(const bf16_t *__restrict__ gu, int64_t T, int64_t F, float limit, float alpha, bf16_t *__restrict__ out, int64_t ldo) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, f8 = F >> 3;
+    if (idx >= T * f8) return;
+    const int64_t t = idx / f8, c = (idx - t * f8) << 3;
+    const uint4 gv = *reinterpret_cast<const uint4 *>(gu + t * 2 * F + c), uv = *reinterpret_cast<const uint4 *>(gu + t * 2 * F + F + c);
+    const bf16_t *ge = reinterpret_cast<const bf16_t *>(&gv), *ue = reinterpret_cast<const bf16_t *>(&uv);
+    uint4 ov; bf16_t *oe = reinterpret_cast<bf16_t *>(&ov);
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+        const float g = fminf(ld_f(ge, x), limit), u = fminf(fmaxf(ld_f(ue, x), -limit), limit);
+        st_f(oe, x, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+    }
+    *reinterpret_cast<uint4 *>(out + t * ldo + c) = ov;
 }
 
 template <class YT>
@@ -600,6 +693,19 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
         if (bf16) retention_seq_kernel<R_, bf16_t><<<grid, dim3(256), 0, s>>>(a, b);                 \
         else retention_seq_kernel<R_, float><<<grid, dim3(256), 0, s>>>(a, b);                       \
     } while (0)
+    if (a.D <= 256) {
+        const size_t lds = ((size_t)2 * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
+#define NVR_RETB(R_)                                                                                 \
+    do {                                                                                             \
+        if (bf16) retention_block_kernel<R_, bf16_t><<<grid, dim3(256), lds, s>>>(a, b);             \
+        else retention_block_kernel<R_, float><<<grid, dim3(256), lds, s>>>(a, b);                   \
+    } while (0)
+        if (rows <= 8) NVR_RETB(8);
+        else if (rows <= 16) NVR_RETB(16);
+        else NVR_RETB(32);
+#undef NVR_RETB
+        return launched("retention");
+    }
     if (rows <= 8) NVR_RET(8);
     else if (rows <= 16) NVR_RET(16);
     else if (rows <= 32) NVR_RET(32);
@@ -611,14 +717,18 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
 int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
                    hipStream_t s) {
     if (T == 0) return 0;
-    const dim3 grid((unsigned)T, (unsigned)H);
-    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(64), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, (bf16_t *)out, ldo);
-    else head_norm_gate_kernel<float><<<grid, dim3(64), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, (float *)out, ldo);
+    const dim3 grid((unsigned)T);
+    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, (bf16_t *)out, ldo);
+    else head_norm_gate_kernel<float><<<grid, dim3(256), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, (float *)out, ldo);
     return launched("head_norm_gate");
 }
 
 int clamped_glu(const void *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s) {
     if (T * F == 0) return 0;
+    if (bf16 && F % 8 == 0 && ldo % 8 == 0 && ((uintptr_t)gu | (uintptr_t)out) % 16 == 0) {
+        clamped_glu8_kernel<<<dim3((unsigned)((T * (F / 8) + 255) / 256)), dim3(256), 0, s>>>((const bf16_t *)gu, T, F, limit, alpha, (bf16_t *)out, ldo);
+        return launched("clamped_glu");
+    }
     const dim3 grid((unsigned)((T * F + 255) / 256));
     if (bf16) clamped_glu_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)gu, T, F, limit, alpha, (bf16_t *)out, ldo);
     else clamped_glu_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)gu, T, F, limit, alpha, (float *)out, ldo);

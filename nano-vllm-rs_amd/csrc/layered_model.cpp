@@ -39,7 +39,7 @@ inline float src_at(int dtype, const void *src, size_t i) {
 }  // namespace
 
 LayeredModel::~LayeredModel() {
-    for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq, (void *)w.pen})
+    for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq, (void *)w.sin_t, (void *)w.pen})
         if (p) (void)hipFree(p);
     for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
     if (attn_ws) (void)hipFree(attn_ws);
@@ -88,11 +88,21 @@ int LayeredModel::init(nvr_model_runner &r) {
             if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
             for (float **p : {&w.r1, &w.r2, &w.sink}) { RC(dmalloc(p, (size_t)L.heads * 4)); NVR_HIP_CHECK(hipMemset(*p, 0, (size_t)L.heads * 4)); }
         } else {
-            std::vector<float> d(L.heads), f((size_t)std::max<int64_t>(L.rot_dims / 2, 1));
+            std::vector<float> d(L.heads);
             for (int64_t h = 0; h < L.heads; ++h) d[(size_t)h] = (float)L.decay[(size_t)h];
-            for (int64_t j = 0; j < L.rot_dims / 2; ++j) f[(size_t)j] = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
             RC(dmalloc(&w.decay, d.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.decay, d.data(), d.size() * 4, hipMemcpyHostToDevice));
-            RC(dmalloc(&w.freq, f.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.freq, f.data(), f.size() * 4, hipMemcpyHostToDevice));
+            // rotation table: the angle is the f32 product of the position and the f32 frequency; its cosine and sine are rounded once from f64
+            const int64_t half = L.rot_dims / 2;
+            std::vector<float> cs((size_t)std::max<int64_t>(r.max_pos * half, 1)), sn(cs.size());
+            for (int64_t j = 0; j < half; ++j) {
+                const float f = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
+                for (int64_t p = 0; p < r.max_pos; ++p) {
+                    const float ang = (float)p * f;
+                    cs[(size_t)(p * half + j)] = (float)std::cos((double)ang); sn[(size_t)(p * half + j)] = (float)std::sin((double)ang);
+                }
+            }
+            RC(dmalloc(&w.freq, cs.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.freq, cs.data(), cs.size() * 4, hipMemcpyHostToDevice));
+            RC(dmalloc(&w.sin_t, sn.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.sin_t, sn.data(), sn.size() * 4, hipMemcpyHostToDevice));
         }
         max_nmix = std::max(max_nmix, w.nmix); max_kcat = std::max(max_kcat, w.kcat); max_hv = std::max(max_hv, hv);
         if (L.has_mlp) max_ff = std::max(max_ff, L.ff);
@@ -338,7 +348,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
                 RC(kl::sink_attention(a, b, bf16, s));
         } else {
             kl::RetentionArgs a{};
-            a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.freq = w.freq; a.rot_dims = (int32_t)L.rot_dims;
+            a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.cos_t = w.freq; a.sin_t = w.sin_t; a.rot_dims = (int32_t)L.rot_dims;
             a.kscale = 1.0f / std::sqrt((float)L.dim); a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.state = st.state; a.o = ret_o;
             RC(kl::retention(a, b, bf16, s));
             RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, cat, w.kcat, bf16, s));

@@ -45,7 +45,7 @@ public:
     struct LayerW {
         void *mix = nullptr, *gu = nullptr, *out = nullptr; // [Nmix][W], [2 ff][W], [W][Kcat] (mixer output columns, then feed-forward columns)
         float *canon1 = nullptr, *canon2 = nullptr;         // [W][taps]
-        float *r1 = nullptr, *r2 = nullptr, *sink = nullptr, *decay = nullptr, *freq = nullptr;
+        float *r1 = nullptr, *r2 = nullptr, *sink = nullptr, *decay = nullptr, *freq = nullptr, *sin_t = nullptr;   // freq: the cosine table, sin_t: the sines ([positions][rot_dims / 2])
         float g1 = 1.f, g2 = 1.f;
         float *pen = nullptr; bool pen_dirty = true;        // attention on the matrix cores: r1 * ln(1 + r2 * d) by head and distance
         int64_t nmix = 0, kcat = 0, mixcols = 0;            // rows of mix, columns of out, of which the mixer's
