@@ -539,7 +539,6 @@ __global__ __launch_bounds__(256) void clamped_glu_kernel(const OT *__restrict__
     st_f(out, t * ldo + c, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
 }
 
-template <class YT>
 // the same, 8 bf16 elements (16 bytes) per thread: F and ldo multiples of 8
 __global__ __launch_bounds__(256) void clamped_glu8_kernel(const bf16_t *__restrict__ gu, int64_t T, int64_t F, float limit, float alpha, bf16_t *__restrict__ out, int64_t ldo) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, f8 = F >> 3;
