@@ -39,6 +39,7 @@ inline float src_at(int dtype, const void *src, size_t i) {
 }  // namespace
 
 LayeredModel::~LayeredModel() {
+    for (auto &g : graphs) if (g.second) (void)hipGraphExecDestroy(g.second);
     for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq, (void *)w.sin_t, (void *)w.pen})
         if (p) (void)hipFree(p);
     for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
@@ -264,6 +265,8 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
     if ((int64_t)R > logit_rows_cap) {                                   // (grown outside any capture: an allocation synchronises)
         NVR_HIP_CHECK(hipStreamSynchronize(r.stream));
         (void)hipFree(r.logits); r.logits = nullptr;
+        for (auto &g : graphs) if (g.second) (void)hipGraphExecDestroy(g.second);   // (they hold the old address)
+        graphs.clear();
         logit_rows_cap = (int64_t)R;
         NVR_HIP_CHECK(hipMalloc((void **)&r.logits, (size_t)(logit_rows_cap * spec.vocab * 4)));
     }
@@ -314,6 +317,49 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
     b.T = (int32_t)T; b.B = (int32_t)nseq; b.max_ctx = (int32_t)max_ctx; b.max_rows = (int32_t)max_rows;
     const int32_t *d_want = (const int32_t *)(in_dev + o_want);
 
+    StepPlan plan{b, d_want, (int64_t)R, T, max_ctx, o_tiles, n_tiles};
+    bool decode_sized = !r.cfg.enforce_eager;
+    for (size_t i = 0; i < nseq && decode_sized; ++i) decode_sized = seqs[i]->chunk_len == 1;
+    if (decode_sized) {
+        const int64_t bucket = (max_ctx + 255) / 256 * 256;
+        plan.max_ctx = plan.b.max_ctx = (int32_t)bucket;
+        const uint64_t key = ((uint64_t)nseq << 40) | ((uint64_t)R << 20) | (uint64_t)(bucket / 256);
+        auto it = graphs.find(key);
+        if (it == graphs.end()) {
+            if (graphs.size() >= (size_t)r.env.max_graphs) {
+                NVR_HIP_CHECK(hipStreamSynchronize(r.stream));
+                for (auto &g : graphs) if (g.second) (void)hipGraphExecDestroy(g.second);
+                graphs.clear();
+            }
+            graphs.emplace(key, nullptr);                                  // seen once: this step runs eagerly
+            RC(forward(r, plan));
+        } else {
+            if (!it->second) {
+                hipGraph_t g = nullptr; hipGraphExec_t ge = nullptr;
+                NVR_HIP_CHECK(hipStreamBeginCapture(r.stream, hipStreamCaptureModeThreadLocal));
+                int rc = forward(r, plan);
+                hipError_t e = hipStreamEndCapture(r.stream, &g);
+                if (!rc && e != hipSuccess) rc = fail(NVR_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+                if (!rc && hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) != hipSuccess) rc = fail(NVR_ERR_HIP, "hipGraphInstantiate failed");
+                if (g) (void)hipGraphDestroy(g);
+                if (rc) return rc;
+                it->second = ge;
+            }
+            NVR_HIP_CHECK(hipGraphLaunch(it->second, r.stream));
+            ++graph_replays;
+        }
+    } else
+        RC(forward(r, plan));
+    for (size_t i = 0; i < nseq; ++i) slot_par[(size_t)seqs[i]->state_slot] ^= 1;
+    r.last_rows = R; r.last_tokens = T;
+    return NVR_OK;
+}
+
+int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
+    const kl::Batch &b = p.b;
+    const int32_t *d_want = p.d_want;
+    const int64_t T = p.T, R = p.R, max_ctx = p.max_ctx;
+    const std::vector<size_t> &o_tiles = p.o_tiles; const std::vector<int32_t> &n_tiles = p.n_tiles;
     hipStream_t s = r.stream;
     const int64_t W = spec.width;
     const float eps = (float)spec.eps;
@@ -361,10 +407,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
         RC(kl::axpy(x, tmp, bf16, (float)spec.residual_mult, T * W, s));
     }
     RC(kl::norm_rows(x, d_want, (int64_t)R, W, eps, gfinal, xsel, bf16, s));
-    RC(gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits, true));
-    for (size_t i = 0; i < nseq; ++i) slot_par[(size_t)seqs[i]->state_slot] ^= 1;
-    r.last_rows = R; r.last_tokens = T;
-    return NVR_OK;
+    return gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits, true);
 }
 
 }  // namespace nvr

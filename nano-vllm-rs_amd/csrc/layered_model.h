@@ -8,6 +8,7 @@
 // logits buffer and the samplers.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <map>
 #include <string>
 #include <vector>
 #include "json.h"
@@ -64,6 +65,11 @@ public:
     // step inputs
     char *in_host = nullptr, *in_dev = nullptr; size_t in_bytes = 0;
     int64_t logit_rows_cap = 0;
+    // decode-sized steps (one token per sequence) replay a captured hipGraph per (sequences, rows of logits, 256-token context bucket): the step's inputs
+    // live at fixed places of the device arena, so a replay differs from its capture only in what the upload put there.  A key is captured the second
+    // time it is seen (its first step also builds what is built once: penalty tables)
+    std::map<uint64_t, hipGraphExec_t> graphs;
+    uint64_t graph_replays = 0;
 
     ~LayeredModel();
     int init(nvr_model_runner &r);
@@ -71,6 +77,8 @@ public:
     int load_tensor(nvr_model_runner &r, const char *name, int dtype, const int64_t *shape, int ndim, const void *data);
 
 private:
+    struct StepPlan { kl::Batch b; const int32_t *d_want; int64_t R, T, max_ctx; std::vector<size_t> o_tiles; std::vector<int32_t> n_tiles; };
+    int forward(nvr_model_runner &r, const StepPlan &p);
     int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);
 };

@@ -8,7 +8,8 @@ import sys
 
 # in-process tensor-parallel tests drive up to 8 ranks of one process on one GPU, each on its own stream, and their one-shot
 # collectives wait for each other INSIDE kernels: every stream needs a hardware queue of its own (HIP's default is 4 per process)
-os.environ.setdefault("GPU_MAX_HW_QUEUES", "16")
+# (set, not defaulted: a box that exports HIP's own default of 4 would leave 8 in-process ranks on 4 queues, and their in-kernel waits would never meet)
+os.environ["GPU_MAX_HW_QUEUES"] = "16"
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:

@@ -9,7 +9,7 @@ DOCS = ["DESIGN.md", "INTEGRATION.md", "README.md"]
 # not C-ABI symbols: the package / library / handle-type / python-module names that share the prefix
 NOT_SYMBOLS = {"nvr_import", "nvr_oracle", "nvr_api", "nvr_config", "nvr_model_config", "nvr_sampling_params", "nvr_attn_meta", "nvr_step_info", "nvr_status",
                "nvr_seq", "nvr_engine", "nvr_scheduler", "nvr_model_runner", "nvr_block_manager", "nvr_local_group", "nvr_sequence_output", "nvr_sched_stats",
-               "nvr_bm_stats", "nvr_engine_stats", "nvr_health_status", "nvr_half", "nvr_stream_fn", "nvr_pmc"}
+               "nvr_bm_stats", "nvr_engine_stats", "nvr_health_status", "nvr_half", "nvr_stream_fn", "nvr_pmc", "nvr_model_spec"}
 
 
 def _header_symbols():
@@ -53,7 +53,7 @@ def test_every_cited_abi_symbol_and_test_name_exists():
         for name, is_prefix in _cited(text, "test_"):
             if name in ("test_", "test_tp", "test_kernels_gpu", "test_engine_gpu", "test_host_parity", "test_oracle_kat", "test_golden", "test_scale", "test_weights",
                         "test_tokenizer", "test_ctrl", "test_bf16_gpu", "test_kernels_bf16_gpu", "test_kernels_f32_gpu", "test_baseline_parity", "test_sanitizers",
-                        "test_bench_counters", "test_design_refs"):
+                        "test_bench_counters", "test_design_refs", "test_rugudra_host", "test_rugudra_gpu"):
                 continue                                                  # file names
             ok = any(t.startswith(name) for t in tests) if is_prefix else name in tests
             if not ok and any(t.startswith(name) for t in tests) and len(name) >= 24:
