@@ -42,6 +42,7 @@ struct FlashParams {
     int32_t nq_total, shared_len, num_parts;
     float *part_o, *part_ml;
     const int32_t *srows, *scount;     // optional: only the rows srows[0 .. *scount) of the batch share the prefix (row srows[0] names its blocks)
+    const float *r1, *r2, *sink; int64_t ldo;   // PEN instantiations: distance penalty and sink per head (FlashArgs); ldo: output row stride in elements
 };
 
 
@@ -121,7 +122,7 @@ constexpr int FLASH_WAVES = NVR_FLASH_WAVES;     // waves per workgroup: 32 quer
 // schedule — 128/G sequences per workgroup, no causal mask, every key of [0, shared_len) visible to every row — and the result
 // leaves as the split-KV partial of partition 0 (unnormalised f32 o, scaled max, sum), merged with the per-sequence remainder
 // by attn_merge_kernel.
-template <int D, int G, bool PAGED, bool UB = false, bool SHARED = false>
+template <int D, int G, bool PAGED, bool UB = false, bool SHARED = false, bool PEN = false>
 __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefill_kernel(FlashParams p) {   // 2 waves per SIMD: <= 256 registers per lane
     constexpr int NT = 64 * FLASH_WAVES;         // threads
     constexpr int KT = NVR_FLASH_KT;             // keys per step
@@ -262,6 +263,15 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
         for (int i = 0; i < NDT; ++i) o[t][i] = (float4_t){0.f, 0.f, 0.f, 0.f};
     }
     const float c2 = p.scale * 1.44269504088896340736f;
+    // PEN: the scores are moved to the base-2 domain before the softmax (s <- s c2 - r1 log2(1 + r2 (i - j)): r1 ln(x) log2(e) = r1 log2(x), one v_log_f32 per
+    // score), so the factor of the exponent is 1 from there on; the sink is the running maximum's first value and a 1 in the running sum
+    const float cs = PEN ? 1.0f : c2;
+    float pr1[NQT], pr2[NQT];
+#pragma unroll
+    for (int t = 0; t < NQT; ++t) {
+        pr1[t] = (PEN && p.r1) ? p.r1[head[t]] : 0.f; pr2[t] = (PEN && p.r2) ? p.r2[head[t]] : 0.f;
+        if (PEN && p.sink) { m[t] = p.sink[head[t]] * 1.44269504088896340736f; ol[t] = (float4_t){1.f, 1.f, 1.f, 1.f}; }
+    }
     half8_t ones;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ones[e] = (half_t)1.0f;
@@ -302,6 +312,17 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
                 for (int t = 0; t < NQT; ++t) s[t][mt] = mfma16(kf[mt & 1][ks], qf[t][ks], s[t][mt]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (PEN) {
+#pragma unroll
+            for (int t = 0; t < NQT; ++t)
+#pragma unroll
+                for (int mt = 0; mt < NMT; ++mt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float dist = (float)max(qpos[t] - (kt + mt * 16 + g4 * 4 + e), 0);
+                        s[t][mt][e] = fmaf(s[t][mt][e], c2, -pr1[t] * __builtin_amdgcn_logf(fmaf(pr2[t], dist, 1.0f)));
+                    }
+        }
         // causal mask only on steps that reach past the tile's first query (keys kt + mt*16 + g4*4 + e)
         if (!SHARED && kt + KT - 1 > tile.pos0) {
 #pragma unroll
@@ -322,15 +343,15 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
             for (int mt = 1; mt < NMT; ++mt) mx = fmaxf(fmaxf(mx, s[t][mt][0]), fmaxf(fmaxf(s[t][mt][1], s[t][mt][2]), s[t][mt][3]));
             mx = max_over_rows(mx);
             const float mn = fmaxf(m[t], mx);                   // finite from the first step on (key 0 <= qpos)
-            alpha[t] = __builtin_amdgcn_exp2f((m[t] - mn) * c2);
+            alpha[t] = __builtin_amdgcn_exp2f((m[t] - mn) * cs);
             moved |= mn != m[t];
             m[t] = mn;
-            const float mc = -mn * c2;
+            const float mc = -mn * cs;
 #pragma unroll
             for (int mt = 0; mt < NMT; ++mt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    pf[t][mt >> 1][(mt & 1) * 4 + e] = (half_t)__builtin_amdgcn_exp2f(fmaf(s[t][mt][e], c2, mc));
+                    pf[t][mt >> 1][(mt & 1) * 4 + e] = (half_t)__builtin_amdgcn_exp2f(fmaf(s[t][mt][e], cs, mc));
         }
         if (__any(moved)) {                                     // wave-uniform: the running max settles after a few steps
 #pragma unroll
@@ -404,7 +425,7 @@ __global__ __launch_bounds__(64 * FLASH_WAVES, 8 / FLASH_WAVES) void flash_prefi
         if (qvalid[t]) {
             const float ls = ol[t][0];                          // every row of the ones-product holds the query's sum
             const float inv = ls > 0.f ? 1.0f / ls : 0.f;
-            half_t *orow = p.out + ((int64_t)qrow[t] * p.H + head[t]) * D + g4 * 4;
+            half_t *orow = p.out + (int64_t)qrow[t] * p.ldo + (int64_t)head[t] * D + g4 * 4;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
                 half4_t hv = {(half_t)(o[t][dt][0] * inv), (half_t)(o[t][dt][1] * inv), (half_t)(o[t][dt][2] * inv), (half_t)(o[t][dt][3] * inv)};
@@ -429,12 +450,17 @@ int flash_prefill(const FlashArgs &a, bool paged, hipStream_t s) {
     p.block_tables = a.block_tables; p.max_blocks = a.max_blocks; p.block_size = a.block_size;
     p.bs_shift = (a.block_size > 0 && (a.block_size & (a.block_size - 1)) == 0) ? __builtin_ctz(a.block_size) : -1;
     p.tiles = a.tiles; p.H = a.H; p.KVH = a.KVH; p.scale = a.scale; p.out = (half_t *)a.out;
+    p.r1 = a.r1; p.r2 = a.r2; p.sink = a.sink; p.ldo = a.ldo ? a.ldo : (int64_t)a.H * a.D;
+    const bool pen = (a.r1 && a.r2) || a.sink;
+    if (pen && !paged) return nvr::fail(NVR_ERR_UNSUPPORTED, "flash_prefill: the penalty / sink form reads K and V through block tables");
     const int G = a.H / a.KVH;
     dim3 grid((unsigned)((int64_t)a.ntiles * a.KVH)), block(64 * FLASH_WAVES);
     const bool ub = paged && p.bs_shift >= 0 && a.block_size % NVR_FLASH_KT == 0;
 #define NVR_FLASH(DD, GG)                                                                             \
     if (a.D == DD && G == GG) {                                                                       \
-        if (ub) flash_prefill_kernel<DD, GG, true, true><<<grid, block, 0, s>>>(p);                   \
+        if (pen && ub) flash_prefill_kernel<DD, GG, true, true, false, true><<<grid, block, 0, s>>>(p);   \
+        else if (pen) flash_prefill_kernel<DD, GG, true, false, false, true><<<grid, block, 0, s>>>(p);   \
+        else if (ub) flash_prefill_kernel<DD, GG, true, true><<<grid, block, 0, s>>>(p);              \
         else if (paged) flash_prefill_kernel<DD, GG, true><<<grid, block, 0, s>>>(p);                 \
         else flash_prefill_kernel<DD, GG, false><<<grid, block, 0, s>>>(p);                           \
     }

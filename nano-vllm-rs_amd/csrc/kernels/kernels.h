@@ -58,6 +58,10 @@ struct FlashArgs {
     const FlashTile *tiles; int32_t ntiles;                // device array
     int32_t H, KVH, D; float scale;
     half_bits *out;                                        // [rows, H, D]
+    // Optional (all zero: plain softmax attention).  A distance penalty and a sink per head: score = q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)), and the
+    // softmax denominator also holds exp(sink[h]) (a term with no key and no value).  r1 / r2 together, sink on its own, each [H] f32 on the device.
+    // ldo: elements between the output rows of consecutive query rows (0: H * D)
+    const float *r1, *r2, *sink; int64_t ldo;
 };
 
 // Config.dtype = "float32": attention arguments of the f32 path (kernels/f32_path.hip)

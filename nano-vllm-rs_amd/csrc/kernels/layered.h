@@ -47,6 +47,7 @@ struct SinkAttnArgs {
     int32_t H, G, D, Dv; float scale;
     void *out; int64_t ldo;
     const float *pen; int32_t pen_n;         // tiled form: penalty_table of this layer ([H][pen_n]; null: no penalty)
+    int32_t v_grouped;                       // tiled form: value pages in groups of 8 keys per column (kv_store's v_grouped), else row-major [.][G][Dv]
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the

@@ -84,6 +84,36 @@ __global__ __launch_bounds__(256) void norm_canon_kernel(const float *__restrict
     const int hrows = taps - 1;
     const float *hin = hist + ((int64_t)par * slots + slot) * hrows * W;
     float *hout = hist + ((int64_t)(par ^ 1) * slots + slot) * hrows * W;
+    if (taps <= 8) {
+        // all rows in one pass: every thread keeps the sums of squares of its columns of the (up to 8) rows, one reduction for all of them
+        __shared__ float red8[4][8];
+        float ss[8];
+#pragma unroll
+        for (int d = 0; d < 8; ++d) ss[d] = 0.f;
+        for (int c = threadIdx.x; c < W; c += 256) {
+#pragma unroll
+            for (int d = 0; d < 8; ++d)
+                if (d < taps) {
+                    float v = 0.f;
+                    if (i - d >= 0) { v = x[(int64_t)(t - d) * W + c]; ss[d] += v * v; }
+                    else if (st + i - d >= 0) v = hin[(int64_t)(hrows + (i - d)) * W + c];      // history row e holds position start - hrows + e
+                    u[(int64_t)d * W + c] = v;
+                }
+        }
+#pragma unroll
+        for (int d = 0; d < 8; ++d) if (d < taps) ss[d] = wave_sum(ss[d]);
+        if ((threadIdx.x & 63) == 0)
+#pragma unroll
+            for (int d = 0; d < 8; ++d) red8[threadIdx.x >> 6][d] = ss[d];
+        __syncthreads();
+        for (int c = threadIdx.x; c < W; c += 256)
+#pragma unroll
+            for (int d = 0; d < 8; ++d)
+                if (d < taps && i - d >= 0) {
+                    const float tot = (red8[0][d] + red8[1][d]) + (red8[2][d] + red8[3][d]);
+                    u[(int64_t)d * W + c] *= 1.0f / sqrtf(tot / (float)W + eps);
+                }
+    } else
     for (int d = 0; d < taps; ++d) {
         float *ud = u + (int64_t)d * W;
         if (i - d >= 0) {
@@ -257,11 +287,13 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
         const int bk = jk < nkeys ? jk / bs : 0, bv = jv < nkeys ? jv / bs : 0;
         const bf16_t *kr = kc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * D;
         const bf16_t *vr = vc + (((int64_t)bt[bv] * bs8 + ((jv - bv * bs) >> 3)) * a.G + kvh) * Dv * 8;
+        const bf16_t *vrow = vc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * Dv;      // row-major pages: the key's own row
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             kreg[x] = uint4{0, 0, 0, 0}; vreg[x] = uint4{0, 0, 0, 0};
             if (jk < nkeys && sch + 4 * x < kch) kreg[x] = *reinterpret_cast<const uint4 *>(kr + (sch + 4 * x) * 8);
-            if (jv < nkeys && vcl + 32 * x < Dv) vreg[x] = *reinterpret_cast<const uint4 *>(vr + (vcl + 32 * x) * 8);
+            if (a.v_grouped) { if (jv < nkeys && vcl + 32 * x < Dv) vreg[x] = *reinterpret_cast<const uint4 *>(vr + (vcl + 32 * x) * 8); }
+            else if (jk < nkeys && sch + 4 * x < (Dv >> 3)) vreg[x] = *reinterpret_cast<const uint4 *>(vrow + (sch + 4 * x) * 8);
         }
     };
     if (z < ntl) request(z * KT);
@@ -272,7 +304,12 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             if (sch + 4 * x < kch) *reinterpret_cast<uint4 *>(Ks + skey * KS + (sch + 4 * x) * 8) = kreg[x];
-            if (vcl + 32 * x < Dv) *reinterpret_cast<uint4 *>(Vg + (vkg * VG + vcl + 32 * x) * 8) = vreg[x];
+            if (a.v_grouped) { if (vcl + 32 * x < Dv) *reinterpret_cast<uint4 *>(Vg + (vkg * VG + vcl + 32 * x) * 8) = vreg[x]; }
+            else if (sch + 4 * x < (Dv >> 3)) {                                  // 8 columns of one key: into the key-group layout, element by element
+                const bf16_t *e = reinterpret_cast<const bf16_t *>(&vreg[x]);
+#pragma unroll
+                for (int y = 0; y < 8; ++y) Vg[((skey >> 3) * VG + (sch + 4 * x) * 8 + y) * 8 + (skey & 7)] = e[y];
+            }
         }
         if (a.pen)
             for (int idx = threadIdx.x; idx < g * 128; idx += 256) {
@@ -635,14 +672,14 @@ int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Bat
 }
 
 bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size) {
-    return bf16 && block_size % 8 == 0 && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
+    return bf16 && (block_size % 8 == 0 || !a.v_grouped) && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
            ((uintptr_t)a.q % 16) == 0 && ((uintptr_t)a.kc % 16) == 0 && ((uintptr_t)a.vc % 16) == 0;
 }
 size_t sink_attention_workspace_bytes(int max_workgroups) { return (size_t)max_workgroups * 64 * (256 + 2) * sizeof(float); }
 
 int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *tiles, int ntiles, int nsplit, void *workspace, size_t workspace_bytes, hipStream_t s) {
     if (ntiles == 0) return 0;
-    if (!sink_attention_tiled_ok(a, true, b.block_size)) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention_tiled: shape outside the matrix-core kernel");
+    if (!sink_attention_tiled_ok(a, true, b.block_size) || (a.v_grouped && b.block_size % 8)) return nvr::fail(NVR_ERR_UNSUPPORTED, "sink_attention_tiled: shape outside the matrix-core kernel");
     if (nsplit < 1) nsplit = 1;
     float *po = nullptr, *pml = nullptr;
     if (nsplit > 1) {
@@ -658,7 +695,8 @@ int sink_attention_tiled(const SinkAttnArgs &a, const Batch &b, const AttnTile *
     else sink_attn_mfma_kernel<256><<<grid, dim3(256), lds, s>>>(a, b, tiles, nsplit, po, pml);
     if (int rc = launched("sink_attention_tiled")) return rc;
     if (nsplit > 1) {
-        sink_attn_merge_kernel<<<dim3((unsigned)ntiles, (unsigned)a.G, 64), dim3(64), 0, s>>>(a, b, tiles, nsplit, po, pml);
+        const int g = a.H / a.G, rows = std::min(64, std::max(1, std::min(64 / g, (int)b.max_rows)) * g);      // rows a tile of this step can hold
+        sink_attn_merge_kernel<<<dim3((unsigned)ntiles, (unsigned)a.G, (unsigned)rows), dim3(64), 0, s>>>(a, b, tiles, nsplit, po, pml);
         return launched("sink_attention merge");
     }
     return 0;

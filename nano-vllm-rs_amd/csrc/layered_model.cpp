@@ -87,6 +87,8 @@ int LayeredModel::init(nvr_model_runner &r) {
         RC(dmalloc(&w.canon2, (size_t)(W * taps * 4))); NVR_HIP_CHECK(hipMemset(w.canon2, 0, (size_t)(W * taps * 4)));
         if (L.mixer == LayeredSpec::ATTENTION) {
             if (std::find(attn_groups.begin(), attn_groups.end(), L.heads / L.kv_heads) == attn_groups.end()) attn_groups.push_back(L.heads / L.kv_heads);
+            w.flash = bf16 && L.dim == L.vdim && nvr::kb::flash_prefill_ok((int)L.dim, (int)L.heads, (int)L.kv_heads) && w.nmix % 8 == 0 && w.kcat % 4 == 0;
+            if (w.flash && std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) == flash_groups.end()) flash_groups.push_back(L.heads / L.kv_heads);
             for (float **p : {&w.r1, &w.r2, &w.sink}) { RC(dmalloc(p, (size_t)L.heads * 4)); NVR_HIP_CHECK(hipMemset(*p, 0, (size_t)L.heads * 4)); }
         } else {
             std::vector<float> d(L.heads);
@@ -153,8 +155,8 @@ int LayeredModel::init(nvr_model_runner &r) {
 
     // step inputs: ids | row_seq | want | cu | start | slot | par | block tables
     in_bytes = (size_t)(MT * 8 + MT * 4 * 2 + (r.max_seqs + 1) * 4 + r.max_seqs * 4 * 3 + r.max_seqs * r.max_blocks_per_seq * 4 + 256) +
-               attn_groups.size() * (size_t)((MT + r.max_seqs) * sizeof(kl::AttnTile) + 16);
-    attn_ws_bytes = kl::sink_attention_workspace_bytes(2 * r.num_cus);
+               (attn_groups.size() + 2 * flash_groups.size()) * (size_t)((MT + r.max_seqs) * sizeof(kl::AttnTile) + 16);
+    attn_ws_bytes = kl::sink_attention_workspace_bytes(4 * r.num_cus);
     NVR_HIP_CHECK(hipMalloc(&attn_ws, attn_ws_bytes));
     NVR_HIP_CHECK(hipHostMalloc((void **)&in_host, in_bytes, hipHostMallocDefault));
     NVR_HIP_CHECK(hipMalloc((void **)&in_dev, in_bytes));
@@ -284,7 +286,24 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
         for (size_t i = 0; i < nseq; ++i) cnt += (seqs[i]->chunk_len + (size_t)pw - 1) / (size_t)pw;
         o_tiles[gi] = carve(cnt * sizeof(kl::AttnTile)); n_tiles[gi] = (int32_t)cnt;
     }
+    std::vector<size_t> o_ftiles(flash_groups.size()); std::vector<int32_t> n_ftiles(flash_groups.size(), 0);
+    for (size_t gi = 0; gi < flash_groups.size(); ++gi) {
+        const int64_t pw = nvr::kb::flash_tile_positions((int)flash_groups[gi], 1);
+        size_t cnt = 0;
+        for (size_t i = 0; i < nseq; ++i) cnt += (seqs[i]->chunk_len + (size_t)pw - 1) / (size_t)pw;
+        o_ftiles[gi] = carve(cnt * sizeof(nvr::kt::FlashTile)); n_ftiles[gi] = (int32_t)cnt;
+    }
     if (off > in_bytes) return fail(NVR_ERR_INVARIANT, "execute_model: step inputs of %zu bytes exceed the arena", off);
+    for (size_t gi = 0; gi < flash_groups.size(); ++gi) {
+        const int64_t pw = nvr::kb::flash_tile_positions((int)flash_groups[gi], 1);
+        nvr::kt::FlashTile *tl = (nvr::kt::FlashTile *)(in_host + o_ftiles[gi]);
+        int64_t row = 0;
+        for (size_t i = 0; i < nseq; ++i) {
+            for (int64_t r0 = 0; r0 < (int64_t)seqs[i]->chunk_len; r0 += pw)
+                *tl++ = nvr::kt::FlashTile{(int32_t)(row + r0), (int32_t)std::min<int64_t>(pw, (int64_t)seqs[i]->chunk_len - r0), (int32_t)((int64_t)seqs[i]->chunk_start + r0), (int32_t)i};
+            row += (int64_t)seqs[i]->chunk_len;
+        }
+    }
     for (size_t gi = 0; gi < attn_groups.size(); ++gi) {
         const int64_t pw = std::max<int64_t>(1, 64 / attn_groups[gi]);
         kl::AttnTile *tl = (kl::AttnTile *)(in_host + o_tiles[gi]);
@@ -317,10 +336,10 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
     b.T = (int32_t)T; b.B = (int32_t)nseq; b.max_ctx = (int32_t)max_ctx; b.max_rows = (int32_t)max_rows;
     const int32_t *d_want = (const int32_t *)(in_dev + o_want);
 
-    StepPlan plan{b, d_want, (int64_t)R, T, max_ctx, o_tiles, n_tiles};
-    bool decode_sized = !r.cfg.enforce_eager;
+    bool decode_sized = true;
     for (size_t i = 0; i < nseq && decode_sized; ++i) decode_sized = seqs[i]->chunk_len == 1;
-    if (decode_sized) {
+    StepPlan plan{b, d_want, (int64_t)R, T, max_ctx, o_tiles, n_tiles, o_ftiles, n_ftiles, decode_sized};
+    if (decode_sized && !r.cfg.enforce_eager) {
         const int64_t bucket = (max_ctx + 255) / 256 * 256;
         plan.max_ctx = plan.b.max_ctx = (int32_t)bucket;
         const uint64_t key = ((uint64_t)nseq << 40) | ((uint64_t)R << 20) | (uint64_t)(bucket / 256);
@@ -374,9 +393,20 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
             a.q = (const char *)proj + (size_t)(w.qcol * esz); a.ldq = w.nmix; a.kc = st.kc; a.vc = st.vc; a.r1 = w.r1; a.r2 = w.r2; a.sink = w.sink;
             a.H = (int32_t)L.heads; a.G = (int32_t)L.kv_heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.scale = (float)L.scale;
             a.out = cat; a.ldo = w.kcat;
+            a.v_grouped = w.flash ? 0 : 1;                                          // (a property of the layer: the pages keep one layout)
             const bool tiled = kl::sink_attention_tiled_ok(a, bf16, (int)r.block_size);   // (a property of the layer's shape: the same answer every step)
-            RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, tiled, s));
-            if (tiled) {
+            RC(kl::kv_store(proj, w.nmix, w.kcol, w.vcol, b, L.kv_heads, L.dim, L.vdim, st.kc, st.vc, bf16, tiled && !w.flash, s));
+            if (w.flash && !p.decode_sized) {
+                // prompts and portions: the dense graph's flash kernel in its penalty / sink form (K and V through the block tables, the step's own rows included)
+                const size_t gi = (size_t)(std::find(flash_groups.begin(), flash_groups.end(), L.heads / L.kv_heads) - flash_groups.begin());
+                nvr::kt::FlashArgs f{};
+                f.q = (const uint16_t *)a.q; f.ldq = w.nmix; f.k = (const uint16_t *)st.kc; f.v = (const uint16_t *)st.vc; f.ldkv = 0;
+                f.block_tables = b.block_tables; f.max_blocks = b.max_blocks; f.block_size = b.block_size;
+                f.tiles = (const nvr::kt::FlashTile *)(in_dev + p.o_ftiles[gi]); f.ntiles = p.n_ftiles[gi];
+                f.H = (int32_t)L.heads; f.KVH = (int32_t)L.kv_heads; f.D = (int32_t)L.dim; f.scale = (float)L.scale; f.out = (uint16_t *)cat;
+                f.r1 = w.r1; f.r2 = w.r2; f.sink = w.sink; f.ldo = w.kcat;
+                RC(nvr::kb::flash_prefill(f, true, s));
+            } else if (tiled) {
                 LayerW &wm = lw[li];
                 if (!wm.pen || wm.pen_dirty) {                                      // the penalties by distance, once per set of r1 / r2
                     if (!wm.pen) RC(dmalloc(&wm.pen, (size_t)(L.heads * r.max_pos * 4)));
@@ -388,7 +418,7 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
                 // decode-sized steps over long contexts: few tiles, many keys each — spread every tile's keys over several workgroups
                 const int64_t wgs = (int64_t)n_tiles[gi] * L.kv_heads;
                 int64_t nsplit = 1;
-                if (wgs < r.num_cus && max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / wgs, (max_ctx + 255) / 256, 16}));
+                if (wgs < r.num_cus && max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(4 * r.num_cus) / wgs, (max_ctx + 127) / 128, 16}));
                 RC(kl::sink_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + o_tiles[gi]), n_tiles[gi], (int)nsplit, attn_ws, attn_ws_bytes, s));
             } else
                 RC(kl::sink_attention(a, b, bf16, s));

@@ -48,6 +48,7 @@ public:
         float *canon1 = nullptr, *canon2 = nullptr;         // [W][taps]
         float *r1 = nullptr, *r2 = nullptr, *sink = nullptr, *decay = nullptr, *freq = nullptr, *sin_t = nullptr;   // freq: the cosine table, sin_t: the sines ([positions][rot_dims / 2])
         float g1 = 1.f, g2 = 1.f;
+        bool flash = false;                                 // attention prompts on the dense graph's flash kernel (penalty / sink form): row-major value pages
         float *pen = nullptr; bool pen_dirty = true;        // attention on the matrix cores: r1 * ln(1 + r2 * d) by head and distance
         int64_t nmix = 0, kcat = 0, mixcols = 0;            // rows of mix, columns of out, of which the mixer's
         int64_t qcol = 0, kcol = 0, vcol = 0, gcol = 0;
@@ -60,6 +61,7 @@ public:
     float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32
     void *proj = nullptr, *gu = nullptr, *tmp = nullptr, *a1 = nullptr, *a2 = nullptr, *cat = nullptr, *xsel = nullptr;   // operand type
     int64_t slots = 0; std::vector<int32_t> slot_par;
+    std::vector<int64_t> flash_groups;                      // distinct H / G of the layers whose prompts take the flash kernel: one FlashTile list per value and step
     std::vector<int64_t> attn_groups;                       // distinct H / G of the attention layers: one list of query tiles per value and step
     void *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // split-key partials of decode-sized steps
     // step inputs
@@ -77,7 +79,8 @@ public:
     int load_tensor(nvr_model_runner &r, const char *name, int dtype, const int64_t *shape, int ndim, const void *data);
 
 private:
-    struct StepPlan { kl::Batch b; const int32_t *d_want; int64_t R, T, max_ctx; std::vector<size_t> o_tiles; std::vector<int32_t> n_tiles; };
+    struct StepPlan { kl::Batch b; const int32_t *d_want; int64_t R, T, max_ctx; std::vector<size_t> o_tiles; std::vector<int32_t> n_tiles;
+                      std::vector<size_t> o_ftiles; std::vector<int32_t> n_ftiles; bool decode_sized; };
     int forward(nvr_model_runner &r, const StepPlan &p);
     int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);

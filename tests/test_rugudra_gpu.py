@@ -27,6 +27,9 @@ MECHANISMS = {
     "attention_grouped_heads": make_config([attention_layer(heads=6, kv_heads=2, dim=32, vdim=16, ff=None)]),
     "attention_one_kv_head_per_head": make_config([attention_layer(heads=3, kv_heads=3, dim=32, vdim=32, scale=0.3, ff=None)]),
     "attention_single_kv_head": make_config([attention_layer(heads=4, kv_heads=1, dim=64, vdim=48, ff=None)]),
+    "attention_64_pairs_of_heads": make_config([attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, ff=None)]),
+    "attention_128_four_heads_per_kv_head": make_config([attention_layer(heads=4, kv_heads=1, dim=128, vdim=128, scale=0.05, ff=None)], width=128),
+    "attention_128_one_head_per_kv_head": make_config([attention_layer(heads=2, kv_heads=2, dim=128, vdim=128, scale=0.07, ff=24)]),
     "retention_full_rotation": make_config([retention_layer(heads=3, dim=32, vdim=16, ff=None)]),
     "retention_partial_rotation": make_config([retention_layer(heads=2, dim=32, vdim=32, rot_dims=12, base=77.0, ff=None)]),
     "retention_no_rotation": make_config([retention_layer(heads=2, dim=16, vdim=40, rot_dims=0, ff=None)]),
@@ -63,7 +66,7 @@ def test_sink_and_penalty_each_change_the_result():
 
 # ------------------------------------------------------------------------------------------------ a model with everything, in portions and batches
 def hybrid(vocab=131, width=96):
-    layers = [attention_layer(heads=4, kv_heads=2, dim=32, vdim=32, ff=64),
+    layers = [attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, ff=64),
               retention_layer(heads=2, dim=32, vdim=16, rot_dims=16, ff=None),
               attention_layer(heads=2, kv_heads=1, dim=64, vdim=32, scale=0.11, ff=80, limit=0.9),
               retention_layer(heads=3, dim=16, vdim=32, ff=48)]
@@ -143,12 +146,13 @@ def probe_model(kind, vocab=61, width=64):
     two tokens' values differ.  No convolution (taps 1): a token's key does not depend on its neighbours.  Attention: a weak penalty and a low sink keep far
     keys alive; retention: decays close to 1."""
     if kind == "attention":
-        cfg = make_config([attention_layer(heads=2, kv_heads=1, dim=32, vdim=32, scale=1.0, ff=None)], vocab=vocab, width=width, taps=1, residual_mult=4.0, embedding_scale=0.25)
+        cfg = make_config([attention_layer(heads=2, kv_heads=1, dim=64, vdim=64, scale=0.5, ff=None)], vocab=vocab, width=width, taps=1, residual_mult=4.0, embedding_scale=0.25)
     else:
         cfg = make_config([retention_layer(heads=2, dim=32, vdim=32, decay=[0.999, 0.9995], rot_dims=0, ff=None)], vocab=vocab, width=width, taps=1, residual_mult=4.0, embedding_scale=0.25)
     w = make_weights(cfg, seed=11)
     rng = np.random.default_rng(12)
-    p = bf16_round(rng.standard_normal((32, width)) * (4.0 / np.sqrt(width)))
+    dk = cfg["layers"][0]["mixer"]["dim"]
+    p = bf16_round(rng.standard_normal((dk, width)) * (4.0 / np.sqrt(width)))
     p[:, width // 2:] = 0.0
     w["embed"][:, :width // 2] = bf16_round(0.1 * w["embed"][:, :width // 2]); w["embed"][7, :width // 2] *= 16.0      # every other token's keys are short
     w["embed"][8, :width // 2] = w["embed"][7, :width // 2]
