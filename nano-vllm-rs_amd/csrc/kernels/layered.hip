@@ -84,36 +84,6 @@ __global__ __launch_bounds__(256) void norm_canon_kernel(const float *__restrict
     const int hrows = taps - 1;
     const float *hin = hist + ((int64_t)par * slots + slot) * hrows * W;
     float *hout = hist + ((int64_t)(par ^ 1) * slots + slot) * hrows * W;
-    if (taps <= 8) {
-        // all rows in one pass: every thread keeps the sums of squares of its columns of the (up to 8) rows, one reduction for all of them
-        __shared__ float red8[4][8];
-        float ss[8];
-#pragma unroll
-        for (int d = 0; d < 8; ++d) ss[d] = 0.f;
-        for (int c = threadIdx.x; c < W; c += 256) {
-#pragma unroll
-            for (int d = 0; d < 8; ++d)
-                if (d < taps) {
-                    float v = 0.f;
-                    if (i - d >= 0) { v = x[(int64_t)(t - d) * W + c]; ss[d] += v * v; }
-                    else if (st + i - d >= 0) v = hin[(int64_t)(hrows + (i - d)) * W + c];      // history row e holds position start - hrows + e
-                    u[(int64_t)d * W + c] = v;
-                }
-        }
-#pragma unroll
-        for (int d = 0; d < 8; ++d) if (d < taps) ss[d] = wave_sum(ss[d]);
-        if ((threadIdx.x & 63) == 0)
-#pragma unroll
-            for (int d = 0; d < 8; ++d) red8[threadIdx.x >> 6][d] = ss[d];
-        __syncthreads();
-        for (int c = threadIdx.x; c < W; c += 256)
-#pragma unroll
-            for (int d = 0; d < 8; ++d)
-                if (d < taps && i - d >= 0) {
-                    const float tot = (red8[0][d] + red8[1][d]) + (red8[2][d] + red8[3][d]);
-                    u[(int64_t)d * W + c] *= 1.0f / sqrtf(tot / (float)W + eps);
-                }
-    } else
     for (int d = 0; d < taps; ++d) {
         float *ud = u + (int64_t)d * W;
         if (i - d >= 0) {
@@ -496,6 +466,29 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
         const int nb = min(TB, n - i0);
         __syncthreads();
         const int dsh = (D & (D - 1)) == 0 ? 31 - __clz(D) : -1;
+        // fully rotated bf16 heads: a thread takes 8 coordinates of the lower half and their partners of the upper half as 16-byte loads
+        const bool fast = sizeof(PT) == 2 && a.rot_dims == D && (half & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0;
+        if (fast) {
+            const int cpt = half >> 3;                                   // 8-coordinate pieces of a half
+            for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
+                const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
+                const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
+                const bf16_t *q = pr + a.qcol + (int64_t)h * D + d0, *k = pr + a.kcol + (int64_t)h * D + d0;
+                const uint4 ql = *reinterpret_cast<const uint4 *>(q), qh = *reinterpret_cast<const uint4 *>(q + half);
+                const uint4 kl = *reinterpret_cast<const uint4 *>(k), kh = *reinterpret_cast<const uint4 *>(k + half);
+                const int64_t p = st + i0 + i;
+                const float *cp = a.cos_t + p * half + d0, *sp = a.sin_t + p * half + d0;
+                const bf16_t *qle = reinterpret_cast<const bf16_t *>(&ql), *qhe = reinterpret_cast<const bf16_t *>(&qh);
+                const bf16_t *kle = reinterpret_cast<const bf16_t *>(&kl), *khe = reinterpret_cast<const bf16_t *>(&kh);
+#pragma unroll
+                for (int y = 0; y < 8; ++y) {
+                    const float cs = cp[y], sn = sp[y];
+                    const float qu = ld_f(qle, y), qv = ld_f(qhe, y), ku = ld_f(kle, y), kv = ld_f(khe, y);
+                    qs[i * D + d0 + y] = qu * cs - qv * sn; qs[i * D + half + d0 + y] = qv * cs + qu * sn;
+                    ks[i * D + d0 + y] = (ku * cs - kv * sn) * a.kscale; ks[i * D + half + d0 + y] = (kv * cs + ku * sn) * a.kscale;
+                }
+            }
+        } else
         for (int idx = threadIdx.x; idx < nb * D; idx += 256) {
             const int i = dsh >= 0 ? idx >> dsh : idx / D, d = idx - i * D;
             const PT *pr = (const PT *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;

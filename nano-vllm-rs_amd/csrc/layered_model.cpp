@@ -418,7 +418,7 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
                 // decode-sized steps over long contexts: few tiles, many keys each — spread every tile's keys over several workgroups
                 const int64_t wgs = (int64_t)n_tiles[gi] * L.kv_heads;
                 int64_t nsplit = 1;
-                if (wgs < r.num_cus && max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(4 * r.num_cus) / wgs, (max_ctx + 127) / 128, 16}));
+                if (wgs < r.num_cus && max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / wgs, (max_ctx + 255) / 256, 16}));
                 RC(kl::sink_attention_tiled(a, b, (const kl::AttnTile *)(in_dev + o_tiles[gi]), n_tiles[gi], (int)nsplit, attn_ws, attn_ws_bytes, s));
             } else
                 RC(kl::sink_attention(a, b, bf16, s));
