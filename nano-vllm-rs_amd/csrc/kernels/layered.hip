@@ -21,6 +21,14 @@ __device__ __forceinline__ void st_f(bf16_t *p, int64_t i, float v) {       // r
     p[i] = (bf16_t)(u >> 16);
 }
 
+__device__ __forceinline__ void st4_f(float *p, int64_t i, const float (&v)[4]) { *reinterpret_cast<float4 *>(p + i) = float4{v[0], v[1], v[2], v[3]}; }
+__device__ __forceinline__ void st4_f(bf16_t *p, int64_t i, const float (&v)[4]) {       // i a multiple of 4: one 8-byte store
+    bf16_t h[4];
+#pragma unroll
+    for (int y = 0; y < 4; ++y) st_f(h, y, v[y]);
+    *reinterpret_cast<uint2 *>(p + i) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -115,6 +123,73 @@ __global__ __launch_bounds__(256) void norm_canon_kernel(const float *__restrict
     if (i == n - 1)                                     // the chunk's last row leaves the history of the next step: positions end - hrows .. end - 1
         for (int d = 0; d < hrows; ++d)
             for (int c = threadIdx.x; c < W; c += 256) hout[(int64_t)(hrows - 1 - d) * W + c] = u[(int64_t)d * W + c];
+}
+
+// The same for widths that are multiples of 4 and up to 8 taps, RB rows per workgroup and nothing staged in LDS: the waves first reduce the rows the group
+// needs (its own and the taps-1 before them) to 1 / rms each, then every thread walks its columns four at a time and gathers, per output row, the taps inputs
+// from the step's rows (L1 / L2 hits: a row is read by up to taps neighbours), the slot's history, or zero.
+template <class OT, int RB>
+__global__ __launch_bounds__(256) void norm_canon_rows_kernel(const float *__restrict__ x, Batch b, int W, float eps, int taps, float g1, const float *__restrict__ w1,
+                                                              OT *__restrict__ out1, float g2, const float *__restrict__ w2, OT *__restrict__ out2,
+                                                              float *__restrict__ hist, int64_t slots) {
+    __shared__ float rinv[RB + 8];
+    __shared__ int rs_i[RB], rs_n[RB], rs_st[RB], rs_par[RB]; __shared__ int64_t rs_slot[RB];
+    const int t0 = blockIdx.x * RB, hrows = taps - 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int k = wave; k < RB + hrows; k += 4) {
+        const int gr = t0 - hrows + k;
+        if (gr < 0 || gr >= b.T) continue;
+        const float4 *xr = reinterpret_cast<const float4 *>(x + (int64_t)gr * W);
+        float ss = 0.f;
+        for (int c = lane; c < (W >> 2); c += 64) { const float4 v = xr[c]; ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w); }
+        ss = wave_sum(ss);
+        if (lane == 0) rinv[k] = 1.0f / sqrtf(ss / (float)W + eps);
+    }
+    if (threadIdx.x < RB && t0 + threadIdx.x < b.T) {
+        const int t = t0 + threadIdx.x, sq = b.row_seq[t], c0 = b.cu[sq];
+        rs_i[threadIdx.x] = t - c0; rs_n[threadIdx.x] = b.cu[sq + 1] - c0; rs_st[threadIdx.x] = b.start[sq]; rs_par[threadIdx.x] = b.par[sq]; rs_slot[threadIdx.x] = b.slot[sq];
+    }
+    __syncthreads();
+    for (int c4 = threadIdx.x * 4; c4 < W; c4 += 1024) {
+        float wa[4][8], wb[4][8];
+#pragma unroll
+        for (int y = 0; y < 4; ++y)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { wa[y][j] = j < taps ? w1[(int64_t)(c4 + y) * taps + j] : 0.f; wb[y][j] = (out2 && j < taps) ? w2[(int64_t)(c4 + y) * taps + j] : 0.f; }
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const int t = t0 + r;
+            if (t >= b.T) break;
+            const int i = rs_i[r], st = rs_st[r];
+            const float *hin = hist + ((int64_t)rs_par[r] * slots + rs_slot[r]) * hrows * W;
+            float *hout = hist + ((int64_t)(rs_par[r] ^ 1) * slots + rs_slot[r]) * hrows * W;
+            const bool last = i == rs_n[r] - 1;
+            float a1[4] = {0.f, 0.f, 0.f, 0.f}, a2[4] = {0.f, 0.f, 0.f, 0.f}, u0[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {                       // tap j weighs the row taps - 1 - j back
+                if (j >= taps) break;
+                const int d = taps - 1 - j;
+                float4 u = float4{0.f, 0.f, 0.f, 0.f};
+                if (i - d >= 0) {
+                    const float ri = rinv[r + hrows - d];
+                    u = *reinterpret_cast<const float4 *>(x + (int64_t)(t - d) * W + c4);
+                    u.x *= ri; u.y *= ri; u.z *= ri; u.w *= ri;
+                } else if (st + i - d >= 0) u = *reinterpret_cast<const float4 *>(hin + (int64_t)(hrows + (i - d)) * W + c4);
+                const float uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int y = 0; y < 4; ++y) {
+                    a1[y] += wa[y][j] * (g1 * uu[y]); a2[y] += wb[y][j] * (g2 * uu[y]);
+                    if (d == 0) u0[y] = uu[y];
+                }
+                if (last && d < hrows) *reinterpret_cast<float4 *>(hout + (int64_t)(hrows - 1 - d) * W + c4) = u;
+            }
+            float o1[4], o2[4];
+#pragma unroll
+            for (int y = 0; y < 4; ++y) { o1[y] = g1 * u0[y] + a1[y]; o2[y] = g2 * u0[y] + a2[y]; }
+            st4_f(out1, (int64_t)t * W + c4, o1);
+            if (out2) st4_f(out2, (int64_t)t * W + c4, o2);
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ K / V rows into the paged caches
@@ -648,6 +723,18 @@ int norm_canon(const float *x, const Batch &b, int64_t W, float eps, int taps, f
                bool bf16, float *hist, int64_t slots, hipStream_t s) {
     if (b.T == 0) return 0;
     if (taps < 1) return nvr::fail(NVR_ERR_INVALID_ARG, "norm_canon: taps %d (at least 1)", taps);
+    if (W % 4 == 0 && taps <= 8 && ((uintptr_t)x | (uintptr_t)hist) % 16 == 0) {
+        // rows per workgroup: many for prompts (the convolution weights of a column are read once per workgroup), few for decode-sized steps (more workgroups)
+#define NVR_NC(RB_)                                                                                                                                       \
+    do {                                                                                                                                                  \
+        const dim3 grid((unsigned)((b.T + RB_ - 1) / RB_));                                                                                               \
+        if (bf16) norm_canon_rows_kernel<bf16_t, RB_><<<grid, dim3(256), 0, s>>>(x, b, (int)W, eps, taps, g1, w1, (bf16_t *)out1, g2, w2, (bf16_t *)out2, hist, slots); \
+        else norm_canon_rows_kernel<float, RB_><<<grid, dim3(256), 0, s>>>(x, b, (int)W, eps, taps, g1, w1, (float *)out1, g2, w2, (float *)out2, hist, slots);        \
+    } while (0)
+        if (b.T >= 4096) NVR_NC(16); else if (b.T >= 64) NVR_NC(4); else NVR_NC(1);
+#undef NVR_NC
+        return launched("norm_canon");
+    }
     const size_t lds = (size_t)taps * (size_t)W * 4;
     if (lds > kMaxLds) return nvr::fail(NVR_ERR_UNSUPPORTED, "norm_canon: %d taps of %ld channels do not fit LDS", taps, (long)W);
     if (bf16) norm_canon_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(256), lds, s>>>(x, b, (int)W, eps, taps, g1, w1, (bf16_t *)out1, g2, w2, (bf16_t *)out2, hist, slots);
