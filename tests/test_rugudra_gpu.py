@@ -210,6 +210,72 @@ def test_wide_heads_of_the_largest_size_class():
         check(Driver(cfg, w, dtype).run_alone(toks, cuts=[100, 3, 1]), want, dtype, dtype)
 
 
+# ------------------------------------------------------------------------------------------------ designs and schedules drawn at random
+def random_design(rng):
+    layers = []
+    for _ in range(int(rng.integers(1, 5))):
+        ff = None if rng.random() < 0.25 else int(rng.choice([24, 40, 64, 96]))
+        if rng.random() < 0.55:
+            heads = int(rng.choice([1, 2, 3, 4, 6, 8]))
+            kv = int(rng.choice([d for d in range(1, heads + 1) if heads % d == 0]))
+            dim = int(rng.choice([16, 32, 64, 128]))
+            vdim = dim if rng.random() < 0.6 else int(rng.choice([16, 32, 48, 64]))
+            layers.append(attention_layer(heads=heads, kv_heads=kv, dim=dim, vdim=vdim, scale=float(rng.uniform(0.5, 1.5)) * dim ** -0.5, ff=ff, limit=float(rng.uniform(0.5, 3.0))))
+        else:
+            heads = int(rng.choice([1, 2, 3, 4]))
+            dim = int(rng.choice([16, 32, 64, 128]))
+            layers.append(retention_layer(heads=heads, dim=dim, vdim=int(rng.choice([8, 16, 32, 64, 96])), decay=[float(x) for x in rng.uniform(0.9, 0.9995, heads)],
+                                          rot_dims=int(rng.choice([0, dim // 2, dim])), base=float(rng.choice([100.0, 10000.0, 1e6])), ff=ff, limit=float(rng.uniform(0.5, 3.0))))
+    n = len(layers)
+    loop = None
+    if rng.random() < 0.6:
+        a = int(rng.integers(0, n)); b = int(rng.integers(a + 1, n + 1))
+        loop = (a, b, int(rng.integers(1, 4)))
+    return make_config(layers, vocab=int(rng.choice([50, 97, 128, 211])), width=int(rng.choice([64, 96, 128, 256])), taps=int(rng.integers(1, 6)), loop=loop,
+                       residual_mult=float(rng.uniform(0.3, 1.0)), embedding_scale=float(rng.uniform(0.3, 1.5)), eps=float(rng.choice([1e-6, 1e-5, 1e-3])))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_design_and_schedule(seed):
+    """A design drawn at random (layer order, head counts, sizes, taps, loop, constants) under a schedule drawn at random: up to four live requests, portions of
+    1 .. 70 tokens, requests that skip steps, pages of 8 or 16 or 64 tokens in a pool that only fits the live ones; float32 and bfloat16 against the restatement."""
+    rng = np.random.default_rng(1000 + seed)
+    cfg = random_design(rng)
+    w = make_weights(cfg, seed=seed)
+    lens = [int(x) for x in rng.integers(1, 160, 6)]
+    toks = {i: tokens_of(n, cfg["vocab"], 50 + i) for i, n in enumerate(lens)}
+    want = {i: expected_logits(cfg, w, t) for i, t in toks.items()}
+    page = int(rng.choice([8, 16, 64]))
+    plan, at, live, nxt = [], {}, [], 0
+    prng = np.random.default_rng(2000 + seed)
+    while nxt < len(lens) or live:
+        while len(live) < 4 and nxt < len(lens) and (not live or prng.random() < 0.6):
+            live.append(nxt); at[nxt] = 0; nxt += 1
+        step = []
+        for i in list(live):
+            if len(live) > 1 and prng.random() < 0.25:
+                continue                                                 # left out of this step
+            n = min(int(prng.choice([1, 1, 2, 3, 7, 16, 33, 70])), lens[i] - at[i])
+            step.append((i, at[i], n)); at[i] += n
+            if at[i] == lens[i]:
+                live.remove(i)
+        if step:
+            plan.append(step)
+    pages = sum((n + page - 1) // page for n in sorted(lens)[-4:]) + 1
+    for dtype in ("float32", "bfloat16"):
+        d = Driver(cfg, w, dtype, page=page, pages=pages, slots=4, max_tokens=4 * 70 + 8, max_len=max(lens) + 1)
+        got = {i: [] for i in toks}
+        done = {i: 0 for i in toks}
+        for step in plan:
+            out = d.step([(str(i), toks[i][a:a + n]) for i, a, n in step])
+            for i, a, n in step:
+                got[i].append(out[str(i)]); done[i] += n
+                if done[i] == lens[i]:
+                    d.end(str(i))
+        for i in toks:
+            check(np.concatenate(got[i]), want[i], dtype, f"seed {seed}, request {i} ({dtype}): {cfg['layers']}")
+
+
 # ------------------------------------------------------------------------------------------------ the engine's own entry point
 @pytest.mark.parametrize("chunked", [0, 1])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
