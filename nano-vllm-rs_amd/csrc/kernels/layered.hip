@@ -518,7 +518,7 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
         for (int r = 0; r < RMAX; ++r) { const int d = part + r * 8; if (d < D) S[(int64_t)d * Dv + c] = s[r]; }
 }
 
-// The same recurrence, 16 tokens per barrier round (key size up to 256): a round brings the rotated q, scaled rotated k and v of its tokens into LDS (cosines
+// The same recurrence, 16 tokens per barrier (key size up to 256): a pass brings the rotated q, scaled rotated k and v of its tokens into LDS (cosines
 // and sines from the position table), every thread then walks the tokens with its rows of the state in registers and leaves its partial outputs in LDS; one
 // barrier later they are summed over the 8 row groups.  Token order and arithmetic per token are those of the token-by-token kernel: the result does not depend
 // on where a prompt is cut.  Thread (c, part) owns rows part * RMAX .. part * RMAX + RMAX - 1 of column c.
