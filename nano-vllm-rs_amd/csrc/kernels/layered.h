@@ -48,6 +48,8 @@ struct SinkAttnArgs {
     void *out; int64_t ldo;
     const float *pen; int32_t pen_n;         // tiled form: penalty_table of this layer ([H][pen_n]; null: no penalty)
     int32_t v_grouped;                       // tiled form: value pages in groups of 8 keys per column (kv_store's v_grouped), else row-major [.][G][Dv]
+    int64_t vld;                             // general form: elements between the value rows of consecutive key/value heads (0: Dv); with vc = kc and vld = D the values
+                                             // are the first Dv numbers of the key rows (one cached row per token serves as key and value)
 };
 int sink_attention(const SinkAttnArgs &a, const Batch &b, bool bf16, hipStream_t s);     // any shape; a context that fits the LDS score buffer
 // The same on the matrix cores (bf16 operands, D % 32 == 0, Dv % 16 == 0, both <= 256, H / G <= 16).  tiles (device, built by the host): tile i covers the
@@ -68,11 +70,15 @@ struct RetentionArgs {
     const float *decay, *cos_t, *sin_t; int32_t rot_dims; float kscale;   // cos_t / sin_t: [positions][rot_dims / 2] of angle = position * freq[i]
     int32_t H, D, Dv;
     float *state; float *o;
+    // gated form (az not null): the decay of token t and key channel d of head h is sigmoid(az[t][h * D + d] + abias[h * D + d])^inv_tau, all in f32 from rows of
+    // the operand type (stride ldz), instead of decay[h]; q is scaled by qscale
+    const void *az; int64_t ldz; const float *abias; float inv_tau, qscale;
 };
 int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s);
-// out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * silu(gate[t][h*Dv + c]); gate: rows of the operand type (stride ldg) from column gcol
-int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
-                   hipStream_t s);
+// out[t][h*Dv + c] = o[t][h][c] / rms(o[t][h][:]) * w[c] * silu(gate[t][h*Dv + c]); gate: rows of the operand type (stride ldg) from column gcol; w (one weight per
+// value column, shared by the heads) may be null
+int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out, int64_t ldo,
+                   bool bf16, hipStream_t s);
 
 // g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gu: rows [T][2*F] of the operand type (gate columns, then up columns)
 int clamped_glu(const void *gu, int64_t T, int64_t F, float limit, float alpha, void *out, int64_t ldo, bool bf16, hipStream_t s);
@@ -85,5 +91,62 @@ int norm_rows(const float *x, const int32_t *rows, int64_t R, int64_t W, float e
 
 // y[T][N] (f32, or the operand type) = a[T][K] . w[N][K]^T for shapes the tiled GEMMs do not take (any T, K, N)
 int gemm_any(const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32, bool bf16, hipStream_t s);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------------------
+// Further blocks (layered_blocks.hip)
+int prepare_blocks();                                   // LDS opt-ins (call once, outside captures)
+
+// x[t] = E[ids[t]] (f32), and the same rows into kept (the first of the kept streams) when not null
+int embed_keep(const void *E, bool bf16, const int64_t *ids, int64_t T, int64_t W, float *x, float *kept, hipStream_t s);
+
+// RMS norm in groups: a row of W numbers is split into `groups` equal consecutive parts, each divided by its own sqrt(mean^2 + eps), the whole times w.
+//   xres null: out rows (operand type, stride ldo) = norm(in rows); in: f32 (in_f32) or operand type, stride ldi; rows (may be null) selects input rows.
+//   xres not null: xres[r] += norm(in[r]) (in: operand type), and with w2 also out[r] = norm(xres[r]) * w2 — the sublayer's output joins the stream and the next
+//   sublayer's input leaves in the same pass.
+struct GroupNormArgs {
+    const void *in; int64_t ldi; bool in_f32; const int32_t *rows; int64_t rows_n, W; int32_t groups; float eps; const float *w;
+    float *xres; const float *w2; void *out; int64_t ldo;
+};
+int group_norm(const GroupNormArgs &a, bool bf16, hipStream_t s);
+
+// Latent attention caches ONE row per token: `rank` numbers of the latent (proj columns col ..., divided by their root mean square, times w) and `rot` numbers of a
+// key part shared by the heads, rotated in pairs (2i, 2i+1) by position * freq[i].  pages: [blocks][block_size][rank + rot] of the operand type.
+int latent_store(const void *proj, int64_t ld, int64_t col, const Batch &b, int64_t rank, int64_t rot, float eps, const float *w, const float *freq, void *pages, bool bf16,
+                 hipStream_t s);
+// The rotated part of the queries: q[t][h * qstride + qcol ...] (rot numbers, pairs (2i, 2i+1)) -> out[t][h * ostride + ocol ...]
+int rotate_heads(const void *q, int64_t ldq, int64_t qstride, int64_t qcol, const Batch &b, int64_t H, int64_t rot, const float *freq, void *out, int64_t ldo, int64_t ostride,
+                 int64_t ocol, bool bf16, hipStream_t s);
+
+// y[t][h * hy + n] = sum_k a[t][h * ha + k] * w[h][n][k] (n < N, k < K; rows of a / y / gate with strides lda / ldy / ldg), times sigmoid(gate[t][h * hg + n]) when gate is not null.
+// One matrix per head: the key expansion folded into the queries (w[h] = Wuk_h^T), the value expansion of the attended latent (w[h] = Wuv_h).
+struct HeadLinearArgs { const void *a; int64_t lda, ha; const void *w; void *y; int64_t ldy, hy; const void *gate; int64_t ldg, hg; int32_t T, H, K, N; };
+int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s);
+
+// Rows grouped by expert: y[r] = w[e] a[r] for off[e] <= r < off[e+1] (w: [groups][N][K]).  With src, row r of a is row src[r] / src_div of the array times rscale[src[r]]
+// (the router's weight on the expert's input).  max_rows: an upper bound of off[groups] known to the host (the offsets stay on the device).
+struct GroupedLinearArgs { const void *a; int64_t lda; const void *w; void *y; int64_t ldy; const int32_t *off; int32_t groups, K, N, max_rows; const int32_t *src; const float *rscale; int32_t src_div; };
+int grouped_linear(const GroupedLinearArgs &a, bool bf16, hipStream_t s);
+
+// out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, N(v) = v / sqrt(mean(v^2) + eps) over the F numbers of a row; coef: 4 floats on the device
+int poly_norm(const void *z, int64_t ldz, int64_t T, int64_t F, float eps, const float *coef, void *out, int64_t ldo, bool bf16, hipStream_t s);
+// out = silu(gate) * up; gu: rows [2 F] (gate columns, then up columns)
+int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s);
+
+// Router of a mixture of experts: logits wr h in f32 (wr: [E][W] f32), the top largest per token -> sel / score (= sigmoid of the logit) [T][top]; then the rows
+// grouped by expert: off [E + 1], order [T top] (place -> token * top + choice), place_of (its inverse).
+int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
+              int32_t *place_of, bool bf16, hipStream_t s);
+// out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null)
+int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s);
+
+// The end of a layer, per row and each part optional: the token input (x += rmsnorm(Wp (gelu_tanh(Wg x) * side_embed[id][ecol .. ecol + dim))) * side_norm), the weighted
+// average over depth (this x becomes kept stream nx - 1; x <- sum_j mix[j] kept[j], kept: [streams][kept_rows][W] f32), and the next layer's first norm of the new x.
+struct LayerTailArgs {
+    float *x; int32_t T, W; float eps; const int64_t *ids;
+    const void *side_embed; int64_t side_ld; int32_t ecol, dim; const void *side_gate, *side_proj; const float *side_norm;
+    float *kept; int64_t kept_rows; int32_t nx; const float *mix;
+    const float *wnext; int32_t groups; void *out;
+};
+int layer_tail(const LayerTailArgs &a, bool bf16, hipStream_t s);
 
 }}  // namespace nvr::kl

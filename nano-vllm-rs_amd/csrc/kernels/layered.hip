@@ -243,13 +243,14 @@ __global__ __launch_bounds__(256) void sink_attn_rows_kernel(SinkAttnArgs a, Bat
     const float inv = 1.0f / sum;
     // values: column c by lanes, keys split over the 256 / CW groups
     float *part = sc + ctx;
+    const int64_t vld = a.vld ? a.vld : a.Dv;           // (values inside the key rows: the latent of latent attention)
     for (int cb = 0; cb < a.Dv; cb += 64) {
         const int c = cb + (threadIdx.x & 63), grp = threadIdx.x >> 6;
         float acc = 0.f;
         if (c < a.Dv)
             for (int j = grp; j < ctx; j += 4) {
                 const int64_t row = (int64_t)bt[j / b.block_size] * b.block_size + j % b.block_size;
-                acc += sc[j] * ld_f(vc, (row * a.G + kvh) * a.Dv + c);
+                acc += sc[j] * ld_f(vc, (row * a.G + kvh) * vld + c);
             }
         part[threadIdx.x] = acc;
         __syncthreads();
@@ -467,14 +468,18 @@ __global__ __launch_bounds__(64) void sink_attn_merge_kernel(SinkAttnArgs a, Bat
 
 // ------------------------------------------------------------------------------------------------ retention, token by token
 // One workgroup per (sequence, head, block of 32 value columns): thread (c, part) keeps rows part, part + 8, ... of column c of the state in registers.
-template <int RMAX, class PT>
+// log(sigmoid(z)) without overflow
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <int RMAX, class PT, bool GATED>
 __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Batch b) {
     __shared__ float qs[2][512], ks[2][512], red[8][32];
+    __shared__ float as[GATED ? 2 : 1][GATED ? 512 : 1];
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
     const int c = cb + (threadIdx.x & 31), part = threadIdx.x >> 5;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
-    const float dec = a.decay[h];
+    const float dec = GATED ? 0.f : a.decay[h];
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dv;
     float s[RMAX];
@@ -493,6 +498,10 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
                 if (d < half) { qv = qv * cs - ld_f(q, d + half) * sn; kv = kv * cs - ld_f(k, d + half) * sn; }
                 else { qv = qv * cs + ld_f(q, d - half) * sn; kv = kv * cs + ld_f(k, d - half) * sn; }
             }
+            if (GATED) {
+                qv *= a.qscale;
+                as[buf][d] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)t * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
+            }
             qs[buf][d] = qv; ks[buf][d] = kv * a.kscale;
         }
         __syncthreads();
@@ -501,7 +510,7 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
             const int d = part + r * 8;
-            if (d < D) { s[r] = dec * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
+            if (d < D) { s[r] = (GATED ? as[buf][d] : dec) * s[r] + ks[buf][d] * v; o += s[r] * qs[buf][d]; }
         }
         red[part][threadIdx.x & 31] = o;
         __syncthreads();
@@ -522,16 +531,18 @@ __global__ __launch_bounds__(256) void retention_seq_kernel(RetentionArgs a, Bat
 // and sines from the position table), every thread then walks the tokens with its rows of the state in registers and leaves its partial outputs in LDS; one
 // barrier later they are summed over the 8 row groups.  Token order and arithmetic per token are those of the token-by-token kernel: the result does not depend
 // on where a prompt is cut.  Thread (c, part) owns rows part * RMAX .. part * RMAX + RMAX - 1 of column c.
-template <int RMAX, class PT>
+// GATED: the decay is per token and key channel, sigmoid(z + bias)^(1/tau) with z from rows of the operand type, and q is scaled by qscale (gated linear attention).
+template <int RMAX, class PT, bool GATED>
 __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, Batch b) {
     constexpr int TB = 16;
     extern __shared__ float rsm[];
     const int D = a.D, Dv = a.Dv, half = a.rot_dims / 2;
     float *qs = rsm, *ks = qs + TB * D, *vs = ks + TB * D, *partial = vs + TB * 32;      // [TB][D], [TB][D], [TB][32], [TB][8][32]
+    float *as = partial + TB * 8 * 32;                                                    // GATED: [TB][D] decays
     const int sq = blockIdx.x, h = blockIdx.y, cb = blockIdx.z * 32;
     const int cl = threadIdx.x & 31, c = cb + cl, part = threadIdx.x >> 5;
     const int r0 = b.cu[sq], n = b.cu[sq + 1] - r0, st = b.start[sq];
-    const float dec = a.decay[h];
+    const float dec = GATED ? 0.f : a.decay[h];
     float *S = a.state + (((int64_t)b.slot[sq] * a.H + h) * D) * Dv;
     const bool live = c < Dv;
     float s[RMAX];
@@ -542,7 +553,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
         __syncthreads();
         const int dsh = (D & (D - 1)) == 0 ? 31 - __clz(D) : -1;
         // fully rotated bf16 heads: a thread takes 8 coordinates of the lower half and their partners of the upper half as 16-byte loads
-        const bool fast = sizeof(PT) == 2 && a.rot_dims == D && (half & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0;
+        const bool fast = !GATED && sizeof(PT) == 2 && a.rot_dims == D && (half & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol) & 7) == 0 && ((uintptr_t)a.proj & 15) == 0;
         if (fast) {
             const int cpt = half >> 3;                                   // 8-coordinate pieces of a half
             for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
@@ -576,6 +587,10 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                 if (d < half) { qv = qv * cs - ld_f(q, d + half) * sn; kv = kv * cs - ld_f(k, d + half) * sn; }
                 else { qv = qv * cs + ld_f(q, d - half) * sn; kv = kv * cs + ld_f(k, d - half) * sn; }
             }
+            if (GATED) {
+                qv *= a.qscale;
+                as[idx] = expf(log_sigmoid(ld_f((const PT *)a.az, (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d) + a.abias[(int64_t)h * D + d]) * a.inv_tau);
+            }
             qs[idx] = qv; ks[idx] = kv * a.kscale;
         }
         for (int idx = threadIdx.x; idx < nb * 32; idx += 256) {
@@ -587,7 +602,12 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             const float v = vs[i * 32 + cl];
             const float *kr = ks + i * D + part * RMAX, *qr = qs + i * D + part * RMAX;
             float o = 0.f;
-            if (D == 8 * RMAX) {
+            if (GATED) {
+                const float *ar = as + i * D + part * RMAX;
+#pragma unroll
+                for (int r = 0; r < RMAX; ++r)
+                    if (part * RMAX + r < D) { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+            } else if (D == 8 * RMAX) {
                 float kk[RMAX], qq[RMAX];
 #pragma unroll
                 for (int r = 0; r < RMAX; r += 4) {
@@ -619,7 +639,7 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
 
 template <class OT>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float *__restrict__ o, const OT *__restrict__ gate, int64_t ldg, int64_t gcol, int H, int Dv,
-                                                             float eps, OT *__restrict__ out, int64_t ldo) {
+                                                             float eps, const float *__restrict__ w, OT *__restrict__ out, int64_t ldo) {
     const int64_t t = blockIdx.x; const int lane = threadIdx.x & 63;
     for (int h = threadIdx.x >> 6; h < H; h += 4) {              // a wave per head
         const float *orow = o + (t * H + h) * Dv;
@@ -629,7 +649,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float *__rest
         const float r = 1.0f / sqrtf(ss / (float)Dv + eps);
         for (int c = lane; c < Dv; c += 64) {
             const float g = ld_f(gate, t * ldg + gcol + (int64_t)h * Dv + c);
-            st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (g / (1.0f + expf(-g))));
+            st_f(out, t * ldo + (int64_t)h * Dv + c, orow[c] * r * (w ? w[c] : 1.0f) * (g / (1.0f + expf(-g))));
         }
     }
 }
@@ -805,17 +825,23 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
     if (a.rot_dims % 2 || a.rot_dims > a.D) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: %d rotated coordinates of %d", a.rot_dims, a.D);
     const dim3 grid((unsigned)b.B, (unsigned)a.H, (unsigned)((a.Dv + 31) / 32));
     const int rows = (a.D + 7) / 8;
+    const bool gated = a.az != nullptr;
+    if (gated && !a.abias) return nvr::fail(NVR_ERR_INVALID_ARG, "retention: gated decays need their bias");
 #define NVR_RET(R_)                                                                                  \
     do {                                                                                             \
-        if (bf16) retention_seq_kernel<R_, bf16_t><<<grid, dim3(256), 0, s>>>(a, b);                 \
-        else retention_seq_kernel<R_, float><<<grid, dim3(256), 0, s>>>(a, b);                       \
+        if (gated) { if (bf16) retention_seq_kernel<R_, bf16_t, true><<<grid, dim3(256), 0, s>>>(a, b);   \
+                     else retention_seq_kernel<R_, float, true><<<grid, dim3(256), 0, s>>>(a, b); }       \
+        else if (bf16) retention_seq_kernel<R_, bf16_t, false><<<grid, dim3(256), 0, s>>>(a, b);     \
+        else retention_seq_kernel<R_, float, false><<<grid, dim3(256), 0, s>>>(a, b);                \
     } while (0)
     if (a.D <= 256) {
-        const size_t lds = ((size_t)2 * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
+        const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
 #define NVR_RETB(R_)                                                                                 \
     do {                                                                                             \
-        if (bf16) retention_block_kernel<R_, bf16_t><<<grid, dim3(256), lds, s>>>(a, b);             \
-        else retention_block_kernel<R_, float><<<grid, dim3(256), lds, s>>>(a, b);                   \
+        if (gated) { if (bf16) retention_block_kernel<R_, bf16_t, true><<<grid, dim3(256), lds, s>>>(a, b);   \
+                     else retention_block_kernel<R_, float, true><<<grid, dim3(256), lds, s>>>(a, b); }       \
+        else if (bf16) retention_block_kernel<R_, bf16_t, false><<<grid, dim3(256), lds, s>>>(a, b); \
+        else retention_block_kernel<R_, float, false><<<grid, dim3(256), lds, s>>>(a, b);            \
     } while (0)
         if (rows <= 8) NVR_RETB(8);
         else if (rows <= 16) NVR_RETB(16);
@@ -831,12 +857,12 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
     return launched("retention");
 }
 
-int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, void *out, int64_t ldo, bool bf16,
-                   hipStream_t s) {
+int head_norm_gate(const float *o, const void *gate, int64_t ldg, int64_t gcol, int64_t T, int64_t H, int64_t Dv, float eps, const float *w, void *out, int64_t ldo,
+                   bool bf16, hipStream_t s) {
     if (T == 0) return 0;
     const dim3 grid((unsigned)T);
-    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, (bf16_t *)out, ldo);
-    else head_norm_gate_kernel<float><<<grid, dim3(256), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, (float *)out, ldo);
+    if (bf16) head_norm_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(o, (const bf16_t *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (bf16_t *)out, ldo);
+    else head_norm_gate_kernel<float><<<grid, dim3(256), 0, s>>>(o, (const float *)gate, ldg, gcol, (int)H, (int)Dv, eps, w, (float *)out, ldo);
     return launched("head_norm_gate");
 }
 

@@ -46,6 +46,14 @@ LayeredModel::~LayeredModel() {
     if (attn_ws) (void)hipFree(attn_ws);
     for (void *p : {embed, head, (void *)x, (void *)proj, (void *)gu, (void *)tmp, (void *)ret_o, a1, a2, cat, xsel, (void *)in_dev}) if (p) (void)hipFree(p);
     if (in_host) (void)hipHostFree(in_host);
+    for (void *p : owned) if (p) (void)hipFree(p);
+}
+
+template <class T> int LayeredModel::own(T **p, size_t bytes) {            // zeroed device memory that lives as long as the model
+    RC(dmalloc(p, bytes));
+    NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
+    owned.push_back((void *)*p);
+    return NVR_OK;
 }
 
 int LayeredModel::init(nvr_model_runner &r) {
@@ -65,11 +73,13 @@ int LayeredModel::init(nvr_model_runner &r) {
     r.device = r.cfg.device_ordinal;
     NVR_HIP_CHECK(hipSetDevice(r.device));
     NVR_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
-    RC(kl::prepare());
+    RC(kl::prepare()); RC(kl::prepare_blocks());
     if (r.f32) RC(nvr::kf::prepare());
     else { RC(nvr::kb::linear_stream_prepare()); RC(nvr::kb::gemm_tiled_prepare()); }
     { int v = 0; if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, r.device) == hipSuccess && v > 0) r.num_cus = v; }
 
+    if (spec.layout == LayeredSpec::SEQUENTIAL) RC(init_sequential(r));
+    else {
     // weights (zero until loaded)
     const int64_t taps = spec.taps;
     int64_t max_nmix = 0, max_ff = 0, max_kcat = 0, max_hv = 0;
@@ -149,6 +159,8 @@ int LayeredModel::init(nvr_model_runner &r) {
     RC(dmalloc(&x, (size_t)(MT * W * 4))); RC(dmalloc(&tmp, (size_t)(MT * W * esz)));
     RC(dmalloc(&proj, (size_t)(MT * max_nmix * esz))); RC(dmalloc(&gu, (size_t)(MT * 2 * max_ff * esz))); RC(dmalloc(&ret_o, (size_t)(MT * max_hv * 4)));
     RC(dmalloc(&a1, (size_t)(MT * W * esz))); RC(dmalloc(&a2, (size_t)(MT * W * esz))); RC(dmalloc(&cat, (size_t)(MT * max_kcat * esz)));
+    }
+    const int64_t MT = r.max_tokens;
     logit_rows_cap = std::max<int64_t>(r.max_seqs, 64);
     RC(dmalloc(&xsel, (size_t)(std::max(MT, logit_rows_cap) * W * esz)));
     RC(dmalloc(&r.logits, (size_t)(logit_rows_cap * V * 4)));
@@ -195,6 +207,7 @@ int LayeredModel::put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t ro
 int LayeredModel::load_tensor(nvr_model_runner &r, const char *name_in, int dtype, const int64_t *shape, int ndim, const void *data) {
     if (dtype < 0 || dtype > 2) return fail(NVR_ERR_INVALID_ARG, "load_tensor: dtype %d", dtype);
     const std::string name(name_in);
+    if (spec.layout == LayeredSpec::SEQUENTIAL) return load_sequential(r, name, dtype, shape, ndim, data);
     const int64_t W = spec.width, V = spec.vocab;
     auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
     auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
@@ -375,6 +388,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
 }
 
 int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
+    if (spec.layout == LayeredSpec::SEQUENTIAL) return forward_sequential(r, p);
     const kl::Batch &b = p.b;
     const int32_t *d_want = p.d_want;
     const int64_t T = p.T, R = p.R, max_ctx = p.max_ctx;
@@ -425,9 +439,10 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
         } else {
             kl::RetentionArgs a{};
             a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.decay = w.decay; a.cos_t = w.freq; a.sin_t = w.sin_t; a.rot_dims = (int32_t)L.rot_dims;
+            a.az = nullptr; a.ldz = 0; a.abias = nullptr; a.inv_tau = 1.f; a.qscale = 1.f;
             a.kscale = 1.0f / std::sqrt((float)L.dim); a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.state = st.state; a.o = ret_o;
             RC(kl::retention(a, b, bf16, s));
-            RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, cat, w.kcat, bf16, s));
+            RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, nullptr, cat, w.kcat, bf16, s));
         }
         if (L.has_mlp) {
             RC(gemm(r, a2, W, w.gu, T, W, 2 * L.ff, gu));
@@ -438,6 +453,284 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
     }
     RC(kl::norm_rows(x, d_want, (int64_t)R, W, eps, gfinal, xsel, bf16, s));
     return gemm(r, xsel, W, head, (int64_t)R, W, spec.vocab, r.logits, true);
+}
+
+// ===================================================================================================================================================
+// Sequential layout: x <- x + nb(mixer(n(x))); x <- x + nb(ff(n(x))); token input; weighted average over depth.
+
+int LayeredModel::init_sequential(nvr_model_runner &r) {
+    const int64_t W = spec.width, V = spec.vocab, MT = r.max_tokens, nL = (int64_t)spec.layers.size();
+    lw.resize(spec.layers.size());
+    int64_t max_nmix = 0, max_q2 = 0, max_qabs = 0, max_ctx = 0, max_hv = 0, max_qlat = 0, max_hd = 0, max_ff = 0, max_rows_e = 0, max_e2f = 0, max_ef = 0;
+    size_t block_bytes = 0;
+    for (size_t i = 0; i < spec.layers.size(); ++i) {
+        const LayeredSpec::Layer &L = spec.layers[i]; LayerW &w = lw[i];
+        const int64_t hv = L.heads * L.vdim, hd = L.heads * L.dim;
+        for (float **p : {&w.n1, &w.n1b}) RC(own(p, (size_t)W * 4));
+        if (L.has_mlp) for (float **p : {&w.n2, &w.n2b}) RC(own(p, (size_t)W * 4));
+        if (L.mixer == LayeredSpec::LATENT) {
+            const int64_t R = L.rot_dim, own_kv = L.kv_from < 0 ? L.kv_rank + R : 0;
+            // mix rows: queries (or their latent), the output gate's rows, the cached row's source
+            w.qcol = 0; const int64_t qn = L.q_rank ? L.q_rank : hd;
+            w.gcol = qn; w.dcol = qn + (L.out_gate ? hv : 0); w.nmix = w.dcol + own_kv;
+            if (L.q_rank) { RC(own(&w.uq, (size_t)(L.heads * (L.dim + R) * L.q_rank * esz))); RC(own(&w.dqn, (size_t)L.q_rank * 4)); max_q2 = std::max(max_q2, L.heads * (L.dim + R)); max_qlat = std::max(max_qlat, L.q_rank); }
+            if (own_kv) { RC(own(&w.dkvn, (size_t)L.kv_rank * 4)); block_bytes += (size_t)(r.block_size * own_kv * esz); }
+            RC(own(&w.ukt, (size_t)(L.heads * L.kv_rank * L.dim * esz))); RC(own(&w.uv, (size_t)(hv * L.kv_rank * esz)));
+            std::vector<float> f((size_t)std::max<int64_t>(R / 2, 1));
+            for (int64_t j = 0; j < R / 2; ++j) f[(size_t)j] = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
+            RC(own(&w.rfreq, f.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.rfreq, f.data(), f.size() * 4, hipMemcpyHostToDevice));
+            max_qabs = std::max(max_qabs, L.heads * (L.kv_rank + R)); max_ctx = std::max(max_ctx, L.heads * L.kv_rank);
+        } else if (L.mixer == LayeredSpec::GLA) {
+            w.qcol = 0; w.kcol = hd; w.vcol = 2 * hd; w.gcol = 2 * hd + hv; w.nmix = 2 * hd + 2 * hv;
+            RC(own(&w.a2b, (size_t)hd * 4)); RC(own(&w.hnorm, (size_t)L.vdim * 4));
+            max_hd = std::max(max_hd, hd);
+        } else return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this mixer does not belong to the sequential layout", i);
+        RC(own(&w.mix, (size_t)(w.nmix * W * esz))); RC(own(&w.wo, (size_t)(W * hv * esz)));
+        if (L.ff_kind == LayeredSpec::FF_POLY) {
+            RC(own(&w.up, (size_t)(L.ff * W * esz))); RC(own(&w.down, (size_t)(W * L.ff * esz))); RC(own(&w.act, 16));
+            max_ff = std::max(max_ff, L.ff);
+        } else if (L.ff_kind == LayeredSpec::FF_MOE) {
+            const int64_t f = L.expert_ff, fs = L.shared_ff;
+            RC(own(&w.router, (size_t)(L.experts * W * 4)));
+            RC(own(&w.egu, (size_t)(L.experts * 2 * f * W * esz))); RC(own(&w.edown, (size_t)(L.experts * W * f * esz)));
+            if (fs) { RC(own(&w.sgu, (size_t)(2 * fs * W * esz))); RC(own(&w.sdown, (size_t)(W * fs * esz))); }
+            max_ff = std::max(max_ff, 2 * fs); max_rows_e = std::max(max_rows_e, L.top); max_e2f = std::max(max_e2f, L.top * 2 * f); max_ef = std::max(max_ef, L.top * f);
+        } else if (L.has_mlp) return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this feed-forward does not belong to the sequential layout", i);
+        if (spec.side_dim) { RC(own(&w.sgate, (size_t)(spec.side_dim * W * esz))); RC(own(&w.sproj, (size_t)(W * spec.side_dim * esz))); RC(own(&w.snorm, (size_t)W * 4)); }
+        RC(own(&w.dwa, (size_t)(i + 2) * 4));                   // (until loaded: the layer's own output passes)
+        { const float one = 1.f; NVR_HIP_CHECK(hipMemcpy(w.dwa + i + 1, &one, 4, hipMemcpyHostToDevice)); }
+        max_nmix = std::max(max_nmix, w.nmix); max_hv = std::max(max_hv, hv);
+    }
+    auto named = [&](void **p, size_t bytes) {              // (the buffers the destructor frees by name)
+        RC(dmalloc((char **)p, bytes));
+        NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
+        return (int)NVR_OK;
+    };
+    RC(named(&embed, (size_t)(V * W * esz))); RC(named(&head, (size_t)(V * W * esz))); RC(own(&wfinal, (size_t)W * 4));
+    if (spec.side_dim) RC(own(&side_embed, (size_t)(V * nL * spec.side_dim * esz)));
+
+    // pages: one row of kv_rank + rot_dim numbers per token for every latent-attention layer with a latent of its own; state per slot for gated linear attention
+    if (r.cfg.num_kvcache_blocks >= 0) r.num_blocks = r.cfg.num_kvcache_blocks;
+    else if (r.cfg.num_kvcache_blocks == -1) r.num_blocks = 1000;
+    else {
+        size_t free_b = 0, total_b = 0;
+        NVR_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        const double budget = (double)free_b - (1.0 - r.cfg.gpu_memory_utilization) * (double)total_b - (double)((nL + 8) * MT * W * 4);
+        const int64_t nb = block_bytes ? (int64_t)(budget * 0.9 / (double)block_bytes) : 1000;
+        if (nb < 1) return fail(NVR_ERR_HIP, "not enough free HBM for one KV block");
+        r.num_blocks = nb;
+    }
+    rs.resize(spec.layers.size());
+    for (size_t i = 0; i < spec.layers.size(); ++i) {
+        const LayeredSpec::Layer &L = spec.layers[i];
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from < 0) RC(own(&rs[i].kc, (size_t)(r.num_blocks * r.block_size * (L.kv_rank + L.rot_dim) * esz)));
+        else if (L.mixer == LayeredSpec::GLA) RC(own(&rs[i].state, (size_t)(slots * L.heads * L.dim * L.vdim * 4)));
+    }
+    for (size_t i = 0; i < spec.layers.size(); ++i) {                           // a layer without a latent of its own reads its source's pages
+        const LayeredSpec::Layer &L = spec.layers[i];
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from >= 0) rs[i].kc = rs[(size_t)L.kv_from].kc;
+    }
+
+    // activations
+    RC(named((void **)&x, (size_t)(MT * W * 4))); RC(own(&kept, (size_t)((nL + 1) * MT * W * 4)));
+    RC(named(&a1, (size_t)(MT * W * esz))); RC(named(&a2, (size_t)(MT * W * esz))); RC(named(&tmp, (size_t)(MT * W * esz)));
+    RC(named(&proj, (size_t)(MT * max_nmix * esz))); RC(named(&cat, (size_t)(MT * max_hv * esz)));
+    RC(own(&qlat, (size_t)(MT * max_qlat * esz))); RC(own(&q2, (size_t)(MT * max_q2 * esz))); RC(own(&qabs, (size_t)(MT * max_qabs * esz))); RC(own(&ctx, (size_t)(MT * max_ctx * esz)));
+    RC(named((void **)&ret_o, (size_t)(MT * max_hv * 4))); RC(own(&az, (size_t)(MT * max_hd * esz)));
+    RC(named(&gu, (size_t)(MT * max_ff * esz))); RC(own(&act, (size_t)(MT * max_ff * esz))); RC(own(&shared_y, (size_t)(MT * W * esz)));
+    RC(own(&e_gu, (size_t)(MT * max_e2f * esz))); RC(own(&e_act, (size_t)(MT * max_ef * esz))); RC(own(&e_y, (size_t)(MT * max_rows_e * W * esz)));
+    RC(own(&moe_i, (size_t)((3 * MT * std::max<int64_t>(max_rows_e, 1) + 1024 + 8) * 4))); RC(own(&moe_score, (size_t)(MT * std::max<int64_t>(max_rows_e, 1) * 4)));
+    return NVR_OK;
+}
+
+// Tensors by the names of the checkpoint: "embed", "head", "final.norm" [W], "side.embed" [vocab][layers * side]; per layer i "l<i>.norm1" / "norm1b" / "norm2" / "norm2b" [W],
+// "l<i>.mix.*" (latent attention: q | dq, dq.norm, uq; dkv, dkv.norm; uk, uv; g; o — gated linear attention: q, k, v, g, o, norm, a1, a2, a2.b), "l<i>.mlp.*" (dense: up, down,
+// act — experts: router, e<j>.{gate,up,down}, shared.{gate,up,down}), "l<i>.side.{gate,proj,norm}", "l<i>.dwa" [i + 2].  Linear weights are [out][in].
+int LayeredModel::load_sequential(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data) {
+    const int64_t W = spec.width, V = spec.vocab, nL = (int64_t)spec.layers.size();
+    const char *name_in = name.c_str();
+    auto is2 = [&](int64_t a, int64_t b) { return ndim == 2 && shape[0] == a && shape[1] == b; };
+    auto bad = [&]() { return fail(NVR_ERR_LEN_MISMATCH, "load_tensor: '%s' has the wrong shape", name_in); };
+    auto unknown = [&]() { return fail(NVR_ERR_UNSUPPORTED, "load_tensor: unknown tensor '%s'", name_in); };
+    auto vec = [&](float *dst, int64_t n) { return (dst && ndim == 1 && shape[0] == n) ? put(r, dst, n, 1, n, dtype, data, false) : bad(); };
+    auto mat = [&](void *dst, int64_t ld, int64_t rows, int64_t cols) { return (dst && is2(rows, cols)) ? put(r, dst, ld, rows, cols, dtype, data, true) : bad(); };
+    auto rows_at = [&](void *base, int64_t row0, int64_t ld) { return (void *)((char *)base + (size_t)(row0 * ld * esz)); };
+    if (name == "embed") return mat(embed, W, V, W);
+    if (name == "head") return mat(head, W, V, W);
+    if (name == "final.norm") return vec(wfinal, W);
+    if (name == "side.embed") return spec.side_dim ? mat(side_embed, nL * spec.side_dim, V, nL * spec.side_dim) : unknown();
+    size_t dot = name.find('.');
+    if (name.size() < 3 || name[0] != 'l' || dot == std::string::npos || dot < 2) return unknown();
+    int64_t li = 0;
+    for (size_t i = 1; i < dot; ++i) { if (name[i] < '0' || name[i] > '9') return unknown(); li = li * 10 + (name[i] - '0'); }
+    if (li >= nL) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: '%s' names a layer the model does not have", name_in);
+    const LayeredSpec::Layer &L = spec.layers[(size_t)li]; LayerW &w = lw[(size_t)li];
+    const std::string rest = name.substr(dot + 1);
+    const int64_t hd = L.heads * L.dim, hv = L.heads * L.vdim, R = L.rot_dim;
+    if (rest == "norm1") return vec(w.n1, W);
+    if (rest == "norm1b") return vec(w.n1b, W);
+    if (rest == "norm2") return L.has_mlp ? vec(w.n2, W) : unknown();
+    if (rest == "norm2b") return L.has_mlp ? vec(w.n2b, W) : unknown();
+    if (rest == "dwa") return vec(w.dwa, li + 2);
+    if (spec.side_dim) {
+        if (rest == "side.gate") return mat(w.sgate, W, spec.side_dim, W);
+        if (rest == "side.proj") return mat(w.sproj, spec.side_dim, W, spec.side_dim);
+        if (rest == "side.norm") return vec(w.snorm, W);
+    }
+    if (rest == "mix.o") return mat(w.wo, hv, W, hv);
+    if (L.mixer == LayeredSpec::LATENT) {
+        if (rest == "mix.q" && !L.q_rank) return mat(w.mix, W, hd, W);
+        if (rest == "mix.dq" && L.q_rank) return mat(w.mix, W, L.q_rank, W);
+        if (rest == "mix.dq.norm" && L.q_rank) return vec(w.dqn, L.q_rank);
+        if (rest == "mix.uq" && L.q_rank) return mat(w.uq, L.q_rank, L.heads * (L.dim + R), L.q_rank);
+        if (rest == "mix.g" && L.out_gate) return mat(rows_at(w.mix, w.gcol, W), W, hv, W);
+        if (rest == "mix.dkv" && L.kv_from < 0) return mat(rows_at(w.mix, w.dcol, W), W, L.kv_rank + R, W);
+        if (rest == "mix.dkv.norm" && L.kv_from < 0) return vec(w.dkvn, L.kv_rank);
+        if (rest == "mix.uv") return mat(w.uv, L.kv_rank, hv, L.kv_rank);
+        if (rest == "mix.uk") {                             // [H D][kv_rank] -> per head its transpose [kv_rank][D]: the expansion folds into the queries
+            if (!is2(hd, L.kv_rank)) return bad();
+            std::vector<float> t((size_t)(hd * L.kv_rank));
+            for (int64_t h = 0; h < L.heads; ++h)
+                for (int64_t k = 0; k < L.dim; ++k)
+                    for (int64_t n = 0; n < L.kv_rank; ++n) t[(size_t)((h * L.kv_rank + n) * L.dim + k)] = src_at(dtype, data, (size_t)((h * L.dim + k) * L.kv_rank + n));
+            return put(r, w.ukt, L.dim, L.heads * L.kv_rank, L.dim, 2, t.data(), true);
+        }
+    } else {
+        if (rest == "mix.q") return mat(rows_at(w.mix, w.qcol, W), W, hd, W);
+        if (rest == "mix.k") return mat(rows_at(w.mix, w.kcol, W), W, hd, W);
+        if (rest == "mix.v") return mat(rows_at(w.mix, w.vcol, W), W, hv, W);
+        if (rest == "mix.g") return mat(rows_at(w.mix, w.gcol, W), W, hv, W);
+        if (rest == "mix.norm") return vec(w.hnorm, L.vdim);
+        if (rest == "mix.a2.b") return vec(w.a2b, hd);
+        if (rest == "mix.a1") {                             // the rank of the decay projection is the tensor's
+            if (ndim != 2 || shape[1] != W || shape[0] < 1 || (w.a_rank && w.a_rank != shape[0])) return bad();
+            w.a_rank = shape[0];
+            if (!w.wa1) RC(own(&w.wa1, (size_t)(w.a_rank * W * esz)));
+            if (w.a_rank > alow_cap) { RC(own(&alow, (size_t)(r.max_tokens * w.a_rank * esz))); alow_cap = w.a_rank; }   // (a smaller one before it stays owned)
+            return put(r, w.wa1, W, w.a_rank, W, dtype, data, true);
+        }
+        if (rest == "mix.a2") {
+            if (ndim != 2 || shape[0] != hd || shape[1] < 1 || (w.a_rank && w.a_rank != shape[1])) return bad();
+            w.a_rank = shape[1];
+            if (!w.wa2) RC(own(&w.wa2, (size_t)(hd * w.a_rank * esz)));
+            return put(r, w.wa2, w.a_rank, hd, w.a_rank, dtype, data, true);
+        }
+    }
+    if (L.ff_kind == LayeredSpec::FF_POLY) {
+        if (rest == "mlp.up") return mat(w.up, W, L.ff, W);
+        if (rest == "mlp.down") return mat(w.down, L.ff, W, L.ff);
+        if (rest == "mlp.act") return vec(w.act, 4);
+    } else if (L.ff_kind == LayeredSpec::FF_MOE) {
+        const int64_t f = L.expert_ff, fs = L.shared_ff;
+        if (rest == "mlp.router") return (is2(L.experts, W)) ? put(r, w.router, W, L.experts, W, dtype, data, false) : bad();
+        if (fs && rest == "mlp.shared.gate") return mat(w.sgu, W, fs, W);
+        if (fs && rest == "mlp.shared.up") return mat(rows_at(w.sgu, fs, W), W, fs, W);
+        if (fs && rest == "mlp.shared.down") return mat(w.sdown, fs, W, fs);
+        if (rest.compare(0, 5, "mlp.e") == 0) {
+            size_t d2 = rest.find('.', 5);
+            if (d2 == std::string::npos || d2 == 5) return unknown();
+            int64_t e = 0;
+            for (size_t i = 5; i < d2; ++i) { if (rest[i] < '0' || rest[i] > '9') return unknown(); e = e * 10 + (rest[i] - '0'); }
+            if (e >= L.experts) return fail(NVR_ERR_UNSUPPORTED, "load_tensor: '%s' names an expert the layer does not have", name_in);
+            const std::string part = rest.substr(d2 + 1);
+            if (part == "gate") return mat(rows_at(w.egu, e * 2 * f, W), W, f, W);
+            if (part == "up") return mat(rows_at(w.egu, e * 2 * f + f, W), W, f, W);
+            if (part == "down") return mat(rows_at(w.edown, e * W, f), f, W, f);
+        }
+    }
+    return unknown();
+}
+
+int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
+    const kl::Batch &b = p.b;
+    const int64_t T = p.T, R = p.R, W = spec.width, nL = (int64_t)spec.layers.size(), MT = r.max_tokens;
+    const float eps = (float)spec.eps; const int groups = (int)spec.norm_groups;
+    hipStream_t s = r.stream;
+    auto at = [&](void *base, int64_t col) { return (void *)((char *)base + (size_t)(col * esz)); };
+    RC(kl::embed_keep(embed, bf16, b.ids, T, W, x, kept, s));
+    {   // the first layer's input; every later one leaves the end of the layer before it
+        kl::GroupNormArgs n{}; n.in = x; n.ldi = W; n.in_f32 = true; n.rows_n = T; n.W = W; n.groups = groups; n.eps = eps; n.w = lw[0].n1; n.out = a1; n.ldo = W;
+        RC(kl::group_norm(n, bf16, s));
+    }
+    for (int64_t i = 0; i < nL; ++i) {
+        const LayeredSpec::Layer &L = spec.layers[(size_t)i]; const LayerW &w = lw[(size_t)i]; RunState &st = rs[(size_t)i];
+        const int64_t hv = L.heads * L.vdim;
+        RC(gemm(r, a1, W, w.mix, T, W, w.nmix, proj));
+        if (L.mixer == LayeredSpec::LATENT) {
+            const int64_t Rr = L.rot_dim, rank = L.kv_rank, Dq = rank + Rr;
+            const void *qsrc = proj; int64_t ldq = w.nmix, qstride = L.dim;
+            if (L.q_rank) {                                 // queries through their own normed latent
+                kl::GroupNormArgs n{}; n.in = proj; n.ldi = w.nmix; n.rows_n = T; n.W = L.q_rank; n.groups = 1; n.eps = eps; n.w = w.dqn; n.out = qlat; n.ldo = L.q_rank;
+                RC(kl::group_norm(n, bf16, s));
+                RC(gemm(r, qlat, L.q_rank, w.uq, T, L.q_rank, L.heads * (L.dim + Rr), q2));
+                qsrc = q2; ldq = L.heads * (L.dim + Rr); qstride = L.dim + Rr;
+            }
+            if (L.kv_from < 0) RC(kl::latent_store(proj, w.nmix, w.dcol, b, rank, Rr, eps, w.dkvn, w.rfreq, st.kc, bf16, s));
+            // the key expansion folded into the queries: per head q' = Wuk_h^T q (kv_rank numbers), then the rotated part
+            kl::HeadLinearArgs ha{}; ha.a = qsrc; ha.lda = ldq; ha.ha = qstride; ha.w = w.ukt; ha.y = qabs; ha.ldy = L.heads * Dq; ha.hy = Dq;
+            ha.T = (int32_t)T; ha.H = (int32_t)L.heads; ha.K = (int32_t)L.dim; ha.N = (int32_t)rank;
+            RC(kl::head_linear(ha, bf16, s));
+            RC(kl::rotate_heads(qsrc, ldq, qstride, L.dim, b, L.heads, Rr, w.rfreq, qabs, L.heads * Dq, Dq, rank, bf16, s));
+            kl::SinkAttnArgs a{};
+            a.q = qabs; a.ldq = L.heads * Dq; a.kc = st.kc; a.vc = st.kc; a.vld = Dq; a.H = (int32_t)L.heads; a.G = 1; a.D = (int32_t)Dq; a.Dv = (int32_t)rank;
+            a.scale = (float)L.scale; a.out = ctx; a.ldo = L.heads * rank;
+            RC(kl::sink_attention(a, b, bf16, s));
+            // the value expansion of the attended latent, and the output gate
+            kl::HeadLinearArgs hu{}; hu.a = ctx; hu.lda = L.heads * rank; hu.ha = rank; hu.w = w.uv; hu.y = cat; hu.ldy = hv; hu.hy = L.vdim;
+            hu.T = (int32_t)T; hu.H = (int32_t)L.heads; hu.K = (int32_t)rank; hu.N = (int32_t)L.vdim;
+            if (L.out_gate) { hu.gate = at(proj, w.gcol); hu.ldg = w.nmix; hu.hg = L.vdim; }
+            RC(kl::head_linear(hu, bf16, s));
+        } else {
+            if (!w.wa1 || !w.wa2) return fail(NVR_ERR_NOT_ALLOCATED, "layer %ld: the decay projections were not loaded", (long)i);
+            RC(gemm(r, a1, W, w.wa1, T, W, w.a_rank, alow));
+            RC(gemm(r, alow, w.a_rank, w.wa2, T, w.a_rank, L.heads * L.dim, az));
+            kl::RetentionArgs a{};
+            a.proj = proj; a.ld = w.nmix; a.qcol = w.qcol; a.kcol = w.kcol; a.vcol = w.vcol; a.rot_dims = 0; a.kscale = 1.0f;
+            a.H = (int32_t)L.heads; a.D = (int32_t)L.dim; a.Dv = (int32_t)L.vdim; a.state = st.state; a.o = ret_o;
+            a.az = az; a.ldz = L.heads * L.dim; a.abias = w.a2b; a.inv_tau = (float)(1.0 / L.tau); a.qscale = 1.0f / std::sqrt((float)L.dim);
+            RC(kl::retention(a, b, bf16, s));
+            RC(kl::head_norm_gate(ret_o, proj, w.nmix, w.gcol, T, L.heads, L.vdim, eps, w.hnorm, cat, hv, bf16, s));
+        }
+        RC(gemm(r, cat, hv, w.wo, T, hv, W, tmp));
+        {   // the mixer's output joins the stream; the feed-forward's input leaves in the same pass
+            kl::GroupNormArgs n{}; n.in = tmp; n.ldi = W; n.rows_n = T; n.W = W; n.groups = groups; n.eps = eps; n.w = w.n1b; n.xres = x;
+            if (L.has_mlp) { n.w2 = w.n2; n.out = a2; n.ldo = W; }
+            RC(kl::group_norm(n, bf16, s));
+        }
+        if (L.ff_kind == LayeredSpec::FF_POLY) {
+            RC(gemm(r, a2, W, w.up, T, W, L.ff, gu));
+            RC(kl::poly_norm(gu, L.ff, T, L.ff, eps, w.act, act, L.ff, bf16, s));
+            RC(gemm(r, act, L.ff, w.down, T, L.ff, W, tmp));
+        } else if (L.ff_kind == LayeredSpec::FF_MOE) {
+            const int64_t f = L.expert_ff, fs = L.shared_ff, n = T * L.top;
+            int32_t *sel = moe_i, *order = sel + MT * L.top, *place_of = order + MT * L.top, *off = place_of + MT * L.top;
+            RC(kl::moe_route(a2, W, T, W, w.router, L.experts, L.top, sel, moe_score, off, order, place_of, bf16, s));
+            kl::GroupedLinearArgs g{}; g.a = a2; g.lda = W; g.w = w.egu; g.y = e_gu; g.ldy = 2 * f; g.off = off; g.groups = (int32_t)L.experts; g.K = (int32_t)W; g.N = (int32_t)(2 * f);
+            g.max_rows = (int32_t)n; g.src = order; g.rscale = moe_score; g.src_div = (int32_t)L.top;
+            RC(kl::grouped_linear(g, bf16, s));
+            RC(kl::silu_mul(e_gu, n, f, e_act, f, bf16, s));
+            kl::GroupedLinearArgs d{}; d.a = e_act; d.lda = f; d.w = w.edown; d.y = e_y; d.ldy = W; d.off = off; d.groups = (int32_t)L.experts; d.K = (int32_t)f; d.N = (int32_t)W; d.max_rows = (int32_t)n;
+            RC(kl::grouped_linear(d, bf16, s));
+            if (fs) {
+                RC(gemm(r, a2, W, w.sgu, T, W, 2 * fs, gu));
+                RC(kl::silu_mul(gu, T, fs, act, fs, bf16, s));
+                RC(gemm(r, act, fs, w.sdown, T, fs, W, shared_y));
+            }
+            RC(kl::moe_combine(e_y, place_of, T, L.top, fs ? shared_y : nullptr, W, tmp, bf16, s));
+        }
+        if (L.has_mlp) {
+            kl::GroupNormArgs n{}; n.in = tmp; n.ldi = W; n.rows_n = T; n.W = W; n.groups = groups; n.eps = eps; n.w = w.n2b; n.xres = x;
+            RC(kl::group_norm(n, bf16, s));
+        }
+        kl::LayerTailArgs t{}; t.x = x; t.T = (int32_t)T; t.W = (int32_t)W; t.eps = eps; t.ids = b.ids;
+        if (spec.side_dim) { t.side_embed = side_embed; t.side_ld = nL * spec.side_dim; t.ecol = (int32_t)(i * spec.side_dim); t.dim = (int32_t)spec.side_dim; t.side_gate = w.sgate; t.side_proj = w.sproj; t.side_norm = w.snorm; }
+        t.kept = kept; t.kept_rows = MT; t.nx = (int32_t)(i + 2); t.mix = w.dwa;
+        if (i + 1 < nL) { t.wnext = lw[(size_t)(i + 1)].n1; t.groups = groups; t.out = a1; }
+        RC(kl::layer_tail(t, bf16, s));
+    }
+    kl::GroupNormArgs n{}; n.in = x; n.ldi = W; n.in_f32 = true; n.rows = p.d_want; n.rows_n = R; n.W = W; n.groups = groups; n.eps = eps; n.w = wfinal; n.out = xsel; n.ldo = W;
+    RC(kl::group_norm(n, bf16, s));
+    return gemm(r, xsel, W, head, R, W, spec.vocab, r.logits, true);
 }
 
 }  // namespace nvr

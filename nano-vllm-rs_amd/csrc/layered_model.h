@@ -1,7 +1,13 @@
 // layered_model.h — models described by their configuration file as a LIST OF LAYERS (the model registry, model_registry.cpp, maps an
-// architecture name either to the dense Qwen3 graph of model_runner.cpp or to this family).  A layer is a token mixer — softmax attention
-// over the paged K/V cache, or retention with a recurrent state — beside an optional feed-forward, both reading the same normalised
-// residual stream; a range of layers can be run several times with the same weights, each pass with a cache / state of its own.
+// architecture name either to the dense Qwen3 graph of model_runner.cpp or to this family).  A layer is a token mixer and an optional feed-forward.
+// Two layouts of a layer:
+//   parallel (Rugudra)   — mixer and feed-forward read the same normalised residual stream (scalar-gain norm + short causal convolution); the mixer is softmax
+//                          attention over paged K/V with a distance penalty and a sink, or retention; a range of layers can run several times with the same
+//                          weights, each pass with a cache / state of its own;
+//   sequential (Pusunex) — x <- x + nb(mixer(n(x))), then x <- x + nb(ff(n(x))) with RMS norms in groups before and after each sublayer; the mixer is latent
+//                          attention (one cached latent row per token, optionally shared with an earlier layer, optionally with a rotated key part and a
+//                          latent for the queries) or gated linear attention; the feed-forward is dense with a polynomial-norm activation or a mixture of
+//                          experts; a per-layer token input and a weighted average over the outputs of all earlier layers close the layer.
 //
 // The family shares the runner's step interface (sequences with a chunk [start, start + len) each: whole prompts, portions of prompts and
 // single decoded tokens in one batch), the block manager's tables (K/V pages) and state slots (recurrent state, convolution history), the
@@ -20,7 +26,9 @@ struct nvr_model_runner;
 namespace nvr {
 
 struct LayeredSpec {
-    enum Mixer { ATTENTION = 0, RETENTION = 1 };
+    enum Mixer { ATTENTION = 0, RETENTION = 1, LATENT = 2, GLA = 3 };
+    enum Ff { FF_NONE = 0, FF_CLAMPED_GLU = 1, FF_POLY = 2, FF_MOE = 3 };
+    enum Layout { PARALLEL = 0, SEQUENTIAL = 1 };
     struct Layer {
         int mixer = ATTENTION;
         int64_t heads = 0, kv_heads = 0, dim = 0, vdim = 0;
@@ -28,7 +36,16 @@ struct LayeredSpec {
         std::vector<double> decay;                          // retention: one per head
         int64_t rot_dims = 0; double rot_base = 10000.0;    // retention: rotated coordinates of q and k
         bool has_mlp = false; int64_t ff = 0; double limit = 0.0;
+        // latent attention: size of the cached latent, of the queries' latent (0: queries straight from the layer's input), of the rotated key part shared by the
+        // heads (0: none; rot_base its frequency base), the layer whose cached rows this layer reads (-1: its own), and whether sigmoid(W_g h) gates the heads' output
+        int64_t kv_rank = 0, q_rank = 0, rot_dim = 0, kv_from = -1; bool out_gate = false;
+        double tau = 1.0;                                   // gated linear attention: decay = sigmoid(z)^(1 / tau)
+        int ff_kind = FF_NONE;
+        int64_t experts = 0, top = 0, expert_ff = 0, shared_ff = 0;   // mixture of experts (shared_ff 0: no shared expert)
     };
+    int layout = PARALLEL;
+    int64_t norm_groups = 1;                                // sequential layout: RMS norms over this many equal parts of a row
+    int64_t side_dim = 0;                                   // per-layer token input: numbers per layer and token (0: none)
     int64_t vocab = 0, width = 0;
     double embedding_scale = 1.0, eps = 1e-5, residual_mult = 1.0;
     int64_t taps = 1;                                       // causal convolution in front of every sublayer (1: a pointwise gain)
@@ -36,6 +53,7 @@ struct LayeredSpec {
     std::vector<int> runs;                                  // layer index of every layer run, in order (loops unrolled)
     bool stateful() const { return true; }                  // convolution history, and recurrent state where there is retention
     static int parse_rugudra(const Json &cfg, LayeredSpec *out);   // (model_registry.cpp)
+    static int parse_pusunex(const Json &cfg, LayeredSpec *out);
 };
 
 class LayeredModel {
@@ -52,11 +70,27 @@ public:
         float *pen = nullptr; bool pen_dirty = true;        // attention on the matrix cores: r1 * ln(1 + r2 * d) by head and distance
         int64_t nmix = 0, kcat = 0, mixcols = 0;            // rows of mix, columns of out, of which the mixer's
         int64_t qcol = 0, kcol = 0, vcol = 0, gcol = 0;
+        // sequential layout
+        float *n1 = nullptr, *n1b = nullptr, *n2 = nullptr, *n2b = nullptr;         // [W] each
+        int64_t dcol = 0;                                   // latent attention: column of the (queries' latent,) cached row's source in the mix projection
+        void *uq = nullptr, *ukt = nullptr, *uv = nullptr, *wo = nullptr;            // [H (D + R)][q_rank]; [H][kv_rank][D] (Wuk per head, transposed); [H][Dv][kv_rank]; [W][H Dv]
+        float *dqn = nullptr, *dkvn = nullptr, *rfreq = nullptr;                     // latent norms' weights, rotation frequencies [rot_dim / 2]
+        void *wa1 = nullptr, *wa2 = nullptr; int64_t a_rank = 0; float *a2b = nullptr, *hnorm = nullptr;   // gated linear attention: decay projections [a_rank][W], [H D][a_rank], bias, head norm [Dv]
+        void *up = nullptr, *down = nullptr; float *act = nullptr;                   // dense feed-forward [ff][W], [W][ff]; 4 coefficients
+        float *router = nullptr; void *egu = nullptr, *edown = nullptr, *sgu = nullptr, *sdown = nullptr;   // [E][W] f32; [E][2 f][W]; [E][W][f]; [2 fs][W]; [W][fs]
+        void *sgate = nullptr, *sproj = nullptr; float *snorm = nullptr, *dwa = nullptr;   // [side][W], [W][side], [W]; [i + 2]
     };
     struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; };
     std::vector<LayerW> lw;
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;
+    // sequential layout
+    float *wfinal = nullptr; void *side_embed = nullptr;                    // [W]; [vocab][layers * side_dim]
+    float *kept = nullptr;                                                  // the embedding output and every layer's output: [layers + 1][max tokens][W] f32
+    void *qlat = nullptr, *q2 = nullptr, *qabs = nullptr, *ctx = nullptr, *alow = nullptr, *az = nullptr, *act = nullptr, *shared_y = nullptr;
+    int64_t alow_cap = 0;
+    void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
+    std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
     // activations
     float *x = nullptr, *ret_o = nullptr;                                  // residual stream, retention outputs: f32
     void *proj = nullptr, *gu = nullptr, *tmp = nullptr, *a1 = nullptr, *a2 = nullptr, *cat = nullptr, *xsel = nullptr;   // operand type
@@ -82,6 +116,10 @@ private:
     struct StepPlan { kl::Batch b; const int32_t *d_want; int64_t R, T, max_ctx; std::vector<size_t> o_tiles; std::vector<int32_t> n_tiles;
                       std::vector<size_t> o_ftiles; std::vector<int32_t> n_ftiles; bool decode_sized; };
     int forward(nvr_model_runner &r, const StepPlan &p);
+    int init_sequential(nvr_model_runner &r);
+    int load_sequential(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
+    int forward_sequential(nvr_model_runner &r, const StepPlan &p);
+    template <class T> int own(T **p, size_t bytes);
     int gemm(nvr_model_runner &r, const void *a, int64_t lda, const void *w, int64_t T, int64_t K, int64_t N, void *y, bool y_f32 = false);
     int put(nvr_model_runner &r, void *dst, int64_t dst_ld, int64_t rows, int64_t cols, int dtype, const void *src, bool as_operand);
 };

@@ -55,10 +55,16 @@ int parse_rugudra_spec(const Json &c, nvr_model_spec *out) {
     return LayeredSpec::parse_rugudra(c, &out->layered);
 }
 
+int parse_pusunex_spec(const Json &c, nvr_model_spec *out) {
+    out->family = 1;
+    return LayeredSpec::parse_pusunex(c, &out->layered);
+}
+
 struct Entry { const char *name; int (*parse)(const Json &, nvr_model_spec *); };
 const Entry kRegistry[] = {
     {"Qwen3ForCausalLM", parse_qwen3},
     {"Rugudra", parse_rugudra_spec},
+    {"Pusunex", parse_pusunex_spec},
 };
 
 }  // namespace
@@ -124,6 +130,80 @@ int LayeredSpec::parse_rugudra(const Json &c, LayeredSpec *s) {
     } else
         for (int64_t i = 0; i < n; ++i) s->runs.push_back((int)i);
     if (s->vocab < 1 || s->width < 1 || s->taps < 1) return fail(NVR_ERR_INVALID_ARG, "config: vocab, width and canon.taps must be positive");
+    return NVR_OK;
+}
+
+// Pusunex: x <- x + nb(mixer(n(x))), x <- x + nb(ff(n(x))) with RMS norms in groups; mixers 'latent_attention' (cached latent, optional 'kv_from' an earlier
+// layer, output gate), 'latent_attention_2' (latent queries, a rotated key part shared by the heads) and 'gla' (gated linear attention); feed-forward 'dense'
+// (polynomial-norm activation) or 'moe' (sigmoid router, top-k, shared expert); a per-layer token input ('token_side') and a weighted average over depth.
+int LayeredSpec::parse_pusunex(const Json &c, LayeredSpec *s) {
+    Reader rd;
+    s->layout = SEQUENTIAL; s->taps = 1; s->embedding_scale = 1.0; s->residual_mult = 1.0;
+    s->vocab = rd.integer(c, "vocab", ""); s->width = rd.integer(c, "width", "");
+    if (const Json *n = rd.need(c, "norm", "")) { s->eps = rd.num(*n, "eps", "norm."); s->norm_groups = rd.integer(*n, "groups", "norm."); }
+    const Json *side = c.get("token_side");
+    s->side_dim = (side && !side->is_null()) ? rd.integer(*side, "dim", "token_side.") : 0;
+    const Json *layers = rd.need(c, "layers", "");
+    if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+    if (layers->kind != Json::Arr || layers->arr.empty()) return fail(NVR_ERR_INVALID_ARG, "config: 'layers' is not a list of layers");
+    if (s->vocab < 1 || s->width < 1 || s->norm_groups < 1 || s->width % s->norm_groups || s->side_dim < 0)
+        return fail(NVR_ERR_INVALID_ARG, "config: vocab and width must be positive, and norm.groups must divide the width");
+    s->layers.clear(); s->runs.clear();
+    for (size_t i = 0; i < layers->arr.size(); ++i) {
+        const Json &lj = layers->arr[i];
+        const std::string w = "layers[" + std::to_string(i) + "].", wm = w + "mixer.";
+        Layer L;
+        const Json *type = rd.need(lj, "type", w), *mx = rd.need(lj, "mixer", w);
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (type->kind != Json::Str) return fail(NVR_ERR_INVALID_ARG, "config: '%stype' is not a string", w.c_str());
+        L.heads = rd.integer(*mx, "heads", wm); L.dim = rd.integer(*mx, "dim", wm); L.vdim = rd.integer(*mx, "vdim", wm);
+        if (type->str == "latent_attention" || type->str == "latent_attention_2") {
+            L.mixer = LATENT; L.kv_heads = 1;
+            L.kv_rank = rd.integer(*mx, "kv_rank", wm); L.scale = rd.num(*mx, "scale", wm);
+            if (type->str == "latent_attention") {
+                L.out_gate = true;
+                const Json *from = mx->get("kv_from");
+                if (from && !from->is_null()) {
+                    L.kv_from = rd.integer(*mx, "kv_from", wm);
+                    if (L.kv_from < 0 || L.kv_from >= (int64_t)i) return fail(NVR_ERR_INVALID_ARG, "config: '%skv_from' must name an earlier layer", w.c_str());
+                    const Layer &src = s->layers[(size_t)L.kv_from];
+                    if (src.mixer != LATENT || src.kv_from >= 0 || src.kv_rank != L.kv_rank || src.rot_dim != 0)
+                        return fail(NVR_ERR_INVALID_ARG, "config: '%skv_from' must name a latent-attention layer with a latent of its own and the same kv_rank", w.c_str());
+                }
+            } else {
+                L.q_rank = rd.integer(*mx, "q_rank", wm); L.rot_dim = rd.integer(*mx, "rot_dim", wm);
+                const Json *rot = rd.need(*mx, "rot", wm);
+                if (rot) {
+                    L.rot_dims = rd.integer(*rot, "dims", wm + "rot."); L.rot_base = rd.num(*rot, "base", wm + "rot.");
+                    if (rd.err.empty() && (L.rot_dims != L.rot_dim || L.rot_dim % 2 || L.rot_dim < 0 || L.q_rank < 1))
+                        return fail(NVR_ERR_INVALID_ARG, "config: %s rotates rot.dims = rot_dim coordinates, an even number, and needs a q_rank", w.c_str());
+                }
+            }
+            if (rd.err.empty() && L.kv_rank < 1) return fail(NVR_ERR_INVALID_ARG, "config: '%skv_rank' must be positive", w.c_str());
+        } else if (type->str == "gla") {
+            L.mixer = GLA; L.kv_heads = L.heads; L.tau = rd.num(*mx, "tau", wm);
+            if (rd.err.empty() && !(L.tau > 0)) return fail(NVR_ERR_INVALID_ARG, "config: '%stau' must be positive", w.c_str());
+        } else return fail(NVR_ERR_UNSUPPORTED, "config: layer type '%s' (latent_attention, latent_attention_2 or gla)", type->str.c_str());
+        const Json *mlp = lj.get("mlp");
+        if (mlp && !mlp->is_null()) {
+            const Json *kind = rd.need(*mlp, "kind", w + "mlp.");
+            if (kind && kind->kind == Json::Str && kind->str == "dense") { L.ff_kind = FF_POLY; L.ff = rd.integer(*mlp, "ff", w + "mlp."); }
+            else if (kind && kind->kind == Json::Str && kind->str == "moe") {
+                L.ff_kind = FF_MOE;
+                const Json *ex = rd.need(*mlp, "expert", w + "mlp."), *ro = rd.need(*mlp, "router", w + "mlp."), *sh = mlp->get("shared");
+                if (ex) L.expert_ff = rd.integer(*ex, "ff", w + "mlp.expert.");
+                if (ro) { L.experts = rd.integer(*ro, "experts", w + "mlp.router."); L.top = rd.integer(*ro, "top", w + "mlp.router."); }
+                if (sh && !sh->is_null()) L.shared_ff = rd.integer(*sh, "ff", w + "mlp.shared.");
+                if (rd.err.empty() && (L.expert_ff < 1 || L.experts < 1 || L.top < 1 || L.top > L.experts || L.shared_ff < 0))
+                    return fail(NVR_ERR_INVALID_ARG, "config: %smlp needs positive expert sizes and 1 <= top <= experts", w.c_str());
+            } else if (kind) return fail(NVR_ERR_UNSUPPORTED, "config: '%smlp.kind' (dense or moe)", w.c_str());
+            L.has_mlp = true;
+            if (rd.err.empty() && L.ff_kind == FF_POLY && L.ff < 1) return fail(NVR_ERR_INVALID_ARG, "config: '%smlp.ff' must be positive", w.c_str());
+        }
+        if (!rd.err.empty()) return fail(NVR_ERR_INVALID_ARG, "%s", rd.err.c_str());
+        if (L.heads < 1 || L.dim < 1 || L.vdim < 1) return fail(NVR_ERR_INVALID_ARG, "config: %s heads, dim and vdim must be positive", w.c_str());
+        s->layers.push_back(L); s->runs.push_back((int)i);
+    }
     return NVR_OK;
 }
 
