@@ -42,7 +42,7 @@ LayeredModel::~LayeredModel() {
     for (auto &g : graphs) if (g.second) (void)hipGraphExecDestroy(g.second);
     for (auto &w : lw) for (void *p : {w.mix, w.gu, w.out, (void *)w.canon1, (void *)w.canon2, (void *)w.r1, (void *)w.r2, (void *)w.sink, (void *)w.decay, (void *)w.freq, (void *)w.sin_t, (void *)w.pen})
         if (p) (void)hipFree(p);
-    for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p) (void)hipFree(p);
+    for (auto &s : rs) for (void *p : {s.kc, s.vc, (void *)s.state, (void *)s.hist}) if (p && !s.borrowed) (void)hipFree(p);
     if (attn_ws) (void)hipFree(attn_ws);
     for (void *p : {embed, head, (void *)x, (void *)proj, (void *)gu, (void *)tmp, (void *)ret_o, a1, a2, cat, xsel, (void *)in_dev}) if (p) (void)hipFree(p);
     if (in_host) (void)hipHostFree(in_host);
@@ -460,6 +460,11 @@ int LayeredModel::forward(nvr_model_runner &r, const StepPlan &p) {
 
 int LayeredModel::init_sequential(nvr_model_runner &r) {
     const int64_t W = spec.width, V = spec.vocab, MT = r.max_tokens, nL = (int64_t)spec.layers.size();
+    auto named = [&](void **p, size_t bytes) {              // (the buffers the destructor frees by name)
+        RC(dmalloc((char **)p, bytes));
+        NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
+        return (int)NVR_OK;
+    };
     lw.resize(spec.layers.size());
     int64_t max_nmix = 0, max_q2 = 0, max_qabs = 0, max_ctx = 0, max_hv = 0, max_qlat = 0, max_hd = 0, max_ff = 0, max_rows_e = 0, max_e2f = 0, max_ef = 0;
     size_t block_bytes = 0;
@@ -485,7 +490,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
             RC(own(&w.a2b, (size_t)hd * 4)); RC(own(&w.hnorm, (size_t)L.vdim * 4));
             max_hd = std::max(max_hd, hd);
         } else return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this mixer does not belong to the sequential layout", i);
-        RC(own(&w.mix, (size_t)(w.nmix * W * esz))); RC(own(&w.wo, (size_t)(W * hv * esz)));
+        RC(named(&w.mix, (size_t)(w.nmix * W * esz))); RC(own(&w.wo, (size_t)(W * hv * esz)));
         if (L.ff_kind == LayeredSpec::FF_POLY) {
             RC(own(&w.up, (size_t)(L.ff * W * esz))); RC(own(&w.down, (size_t)(W * L.ff * esz))); RC(own(&w.act, 16));
             max_ff = std::max(max_ff, L.ff);
@@ -501,11 +506,6 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
         { const float one = 1.f; NVR_HIP_CHECK(hipMemcpy(w.dwa + i + 1, &one, 4, hipMemcpyHostToDevice)); }
         max_nmix = std::max(max_nmix, w.nmix); max_hv = std::max(max_hv, hv);
     }
-    auto named = [&](void **p, size_t bytes) {              // (the buffers the destructor frees by name)
-        RC(dmalloc((char **)p, bytes));
-        NVR_HIP_CHECK(hipMemset(*p, 0, bytes ? bytes : 16));
-        return (int)NVR_OK;
-    };
     RC(named(&embed, (size_t)(V * W * esz))); RC(named(&head, (size_t)(V * W * esz))); RC(own(&wfinal, (size_t)W * 4));
     if (spec.side_dim) RC(own(&side_embed, (size_t)(V * nL * spec.side_dim * esz)));
 
@@ -523,12 +523,12 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
     rs.resize(spec.layers.size());
     for (size_t i = 0; i < spec.layers.size(); ++i) {
         const LayeredSpec::Layer &L = spec.layers[i];
-        if (L.mixer == LayeredSpec::LATENT && L.kv_from < 0) RC(own(&rs[i].kc, (size_t)(r.num_blocks * r.block_size * (L.kv_rank + L.rot_dim) * esz)));
-        else if (L.mixer == LayeredSpec::GLA) RC(own(&rs[i].state, (size_t)(slots * L.heads * L.dim * L.vdim * 4)));
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from < 0) RC(named(&rs[i].kc, (size_t)(r.num_blocks * r.block_size * (L.kv_rank + L.rot_dim) * esz)));
+        else if (L.mixer == LayeredSpec::GLA) RC(named((void **)&rs[i].state, (size_t)(slots * L.heads * L.dim * L.vdim * 4)));
     }
     for (size_t i = 0; i < spec.layers.size(); ++i) {                           // a layer without a latent of its own reads its source's pages
         const LayeredSpec::Layer &L = spec.layers[i];
-        if (L.mixer == LayeredSpec::LATENT && L.kv_from >= 0) rs[i].kc = rs[(size_t)L.kv_from].kc;
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from >= 0) { rs[i].kc = rs[(size_t)L.kv_from].kc; rs[i].borrowed = true; }
     }
 
     // activations

@@ -80,7 +80,7 @@ public:
         float *router = nullptr; void *egu = nullptr, *edown = nullptr, *sgu = nullptr, *sdown = nullptr;   // [E][W] f32; [E][2 f][W]; [E][W][f]; [2 fs][W]; [W][fs]
         void *sgate = nullptr, *sproj = nullptr; float *snorm = nullptr, *dwa = nullptr;   // [side][W], [W][side], [W]; [i + 2]
     };
-    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; };
+    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; };   // borrowed: another run's pages (a shared latent)
     std::vector<LayerW> lw;
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;

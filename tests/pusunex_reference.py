@@ -125,12 +125,17 @@ def gated_expert(h, wt, p):
     return (silu(h @ wt[p + "gate"].T) * (h @ wt[p + "up"].T)) @ wt[p + "down"].T
 
 
-def moe_ff(h, mlp, wt, p):
-    """Sigmoid scores, the `top` largest chosen, the score scales the expert's INPUT; a shared expert for every token."""
+def moe_ff(h, mlp, wt, p, margins=None):
+    """Sigmoid scores, the `top` largest chosen, the score scales the expert's INPUT; a shared expert for every token.  margins (a list) receives, per
+    token, the gap between the last chosen and the first rejected router logit."""
     top = mlp["router"]["top"]
-    s = sigmoid(h @ wt[p + "router"].T)
+    z = h @ wt[p + "router"].T
+    s = sigmoid(z)
     out = np.zeros((h.shape[0], wt[p + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
+        if margins is not None and top < z.shape[1]:
+            zs = np.sort(z[t])[::-1]
+            margins.append(zs[top - 1] - zs[top])
         for e in np.argsort(-s[t], kind="stable")[:top]:
             out[t] += gated_expert(s[t, e] * h[t:t + 1], wt, p + "e%d." % e)[0]
     if mlp.get("shared") is not None:
@@ -144,8 +149,8 @@ def token_side(x, tokens, i, dim, wt, p, side_embed, eps):
     return rms(y, eps) * wt[p + "norm"]
 
 
-def forward(cfg, wt, tokens, layer_outputs=None):
-    """Logits [T, vocab] of one sequence; layer_outputs (a list) receives the stream that leaves every layer."""
+def forward(cfg, wt, tokens, layer_outputs=None, margins=None):
+    """Logits [T, vocab] of one sequence; layer_outputs (a list) receives the stream that leaves every layer, margins the routers' decision gaps."""
     wt = {k: np.asarray(v, dtype=np.float64) for k, v in wt.items()}
     tokens = np.asarray(tokens)
     eps, groups = cfg["norm"]["eps"], cfg["norm"]["groups"]
@@ -166,7 +171,7 @@ def forward(cfg, wt, tokens, layer_outputs=None):
         mlp = L.get("mlp")
         if mlp is not None:
             h = group_norm(x, wt[p + "norm2"], groups, eps)
-            y = poly_ff(h, wt, p + "mlp.", eps) if mlp["kind"] == "dense" else moe_ff(h, mlp, wt, p + "mlp.")
+            y = poly_ff(h, wt, p + "mlp.", eps) if mlp["kind"] == "dense" else moe_ff(h, mlp, wt, p + "mlp.", margins)
             x = x + group_norm(y, wt[p + "norm2b"], groups, eps)
         if cfg.get("token_side") is not None:
             x = x + token_side(x, tokens, i, cfg["token_side"]["dim"], wt, p + "side.", wt["side.embed"], eps)
