@@ -102,10 +102,10 @@ int embed_keep(const void *E, bool bf16, const int64_t *ids, int64_t T, int64_t 
 // RMS norm in groups: a row of W numbers is split into `groups` equal consecutive parts, each divided by its own sqrt(mean^2 + eps), the whole times w.
 //   xres null: out rows (operand type, stride ldo) = norm(in rows); in: f32 (in_f32) or operand type, stride ldi; rows (may be null) selects input rows.
 //   xres not null: xres[r] += norm(in[r]) (in: operand type), and with w2 also out[r] = norm(xres[r]) * w2 — the sublayer's output joins the stream and the next
-//   sublayer's input leaves in the same pass.
+//   sublayer's input leaves in the same pass; with out_plain (and no w2) out[r] = xres[r] itself, in the operand type.
 struct GroupNormArgs {
     const void *in; int64_t ldi; bool in_f32; const int32_t *rows; int64_t rows_n, W; int32_t groups; float eps; const float *w;
-    float *xres; const float *w2; void *out; int64_t ldo;
+    float *xres; const float *w2; void *out; int64_t ldo; bool out_plain;
 };
 int group_norm(const GroupNormArgs &a, bool bf16, hipStream_t s);
 
@@ -139,11 +139,15 @@ int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr,
 // out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null)
 int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s);
 
-// The end of a layer, per row and each part optional: the token input (x += rmsnorm(Wp (gelu_tanh(Wg x) * side_embed[id][ecol .. ecol + dim))) * side_norm), the weighted
+// The per-layer token input is y = Wp (gelu_tanh(Wg x) * E[id][ecol .. ecol + dim)), x += y / rms(y) * wn: two ordinary products with this between them
+// (z = Wg x rows of dim numbers -> g), and its last step inside layer_tail.
+int side_gate(const void *z, const int64_t *ids, const void *E, int64_t lde, int64_t ecol, int64_t dim, int64_t T, void *g, bool bf16, hipStream_t s);
+
+// The end of a layer, per row and each part optional: the token input's last step (x += side_y / rms(side_y) * side_norm; side_y rows of the operand type), the weighted
 // average over depth (this x becomes kept stream nx - 1; x <- sum_j mix[j] kept[j], kept: [streams][kept_rows][W] f32), and the next layer's first norm of the new x.
 struct LayerTailArgs {
-    float *x; int32_t T, W; float eps; const int64_t *ids;
-    const void *side_embed; int64_t side_ld; int32_t ecol, dim; const void *side_gate, *side_proj; const float *side_norm;
+    float *x; int32_t T, W; float eps;
+    const void *side_y; const float *side_norm;
     float *kept; int64_t kept_rows; int32_t nx; const float *mix;
     const float *wnext; int32_t groups; void *out;
 };

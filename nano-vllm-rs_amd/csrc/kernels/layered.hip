@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(SinkAttnArgs a, 
         const int bk = jk < nkeys ? jk / bs : 0, bv = jv < nkeys ? jv / bs : 0;
         const bf16_t *kr = kc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * D;
         const bf16_t *vr = vc + (((int64_t)bt[bv] * bs8 + ((jv - bv * bs) >> 3)) * a.G + kvh) * Dv * 8;
-        const bf16_t *vrow = vc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * Dv;      // row-major pages: the key's own row
+        const bf16_t *vrow = vc + (((int64_t)bt[bk] * bs + (jk - bk * bs)) * a.G + kvh) * (a.vld ? a.vld : (int64_t)Dv);      // row-major pages: the key's own row
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             kreg[x] = uint4{0, 0, 0, 0}; vreg[x] = uint4{0, 0, 0, 0};
@@ -604,9 +604,21 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
             float o = 0.f;
             if (GATED) {
                 const float *ar = as + i * D + part * RMAX;
+                if (D == 8 * RMAX) {
+                    float kk[RMAX], qq[RMAX], aa[RMAX];
 #pragma unroll
-                for (int r = 0; r < RMAX; ++r)
-                    if (part * RMAX + r < D) { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+                    for (int r = 0; r < RMAX; r += 4) {
+                        *reinterpret_cast<float4 *>(kk + r) = *reinterpret_cast<const float4 *>(kr + r);
+                        *reinterpret_cast<float4 *>(qq + r) = *reinterpret_cast<const float4 *>(qr + r);
+                        *reinterpret_cast<float4 *>(aa + r) = *reinterpret_cast<const float4 *>(ar + r);
+                    }
+#pragma unroll
+                    for (int r = 0; r < RMAX; ++r) { s[r] = aa[r] * s[r] + kk[r] * v; o += s[r] * qq[r]; }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < RMAX; ++r)
+                        if (part * RMAX + r < D) { s[r] = ar[r] * s[r] + kr[r] * v; o += s[r] * qr[r]; }
+                }
             } else if (D == 8 * RMAX) {
                 float kk[RMAX], qq[RMAX];
 #pragma unroll
@@ -772,7 +784,7 @@ int kv_store(const void *proj, int64_t ld, int64_t kcol, int64_t vcol, const Bat
 }
 
 bool sink_attention_tiled_ok(const SinkAttnArgs &a, bool bf16, int block_size) {
-    return bf16 && (block_size % 8 == 0 || !a.v_grouped) && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 &&
+    return bf16 && (block_size % 8 == 0 || !a.v_grouped) && a.G >= 1 && a.H % a.G == 0 && a.H / a.G <= 16 && a.D % 32 == 0 && a.Dv % 16 == 0 && a.D <= 256 && a.Dv <= 256 && a.ldq % 8 == 0 && a.vld % 8 == 0 && (!a.vld || !a.v_grouped) &&
            ((uintptr_t)a.q % 16) == 0 && ((uintptr_t)a.kc % 16) == 0 && ((uintptr_t)a.vc % 16) == 0;
 }
 size_t sink_attention_workspace_bytes(int max_workgroups) { return (size_t)max_workgroups * 64 * (256 + 2) * sizeof(float); }

@@ -49,8 +49,8 @@ int launched(const char *what) {
 // sublayer's output joining the residual stream) instead of being stored; with w2 the new residual row is normed once more into out (the next sublayer's input).
 template <class IT, class OT, bool ADD>
 __global__ __launch_bounds__(256) void group_norm_kernel(const IT *__restrict__ in, int64_t ldi, const int32_t *__restrict__ rows, int W, int groups, float eps,
-                                                         const float *__restrict__ w, float *__restrict__ xres, const float *__restrict__ w2, OT *__restrict__ out,
-                                                         int64_t ldo) {
+                                                         const float *__restrict__ w, float *__restrict__ xres, const float *__restrict__ w2, int plain,
+                                                         OT *__restrict__ out, int64_t ldo) {
     const int64_t r = blockIdx.x, src = rows ? rows[r] : r;
     const IT *x = in + src * ldi;
     const int n = W / groups, lane = threadIdx.x & 63;
@@ -64,7 +64,11 @@ __global__ __launch_bounds__(256) void group_norm_kernel(const IT *__restrict__ 
         } else {
             float *xr = xres + r * (int64_t)W;
             float s2 = 0.f;
-            for (int c = lane; c < n; c += 64) { const float v = xr[c0 + c] + ld_f(x, c0 + c) * inv * w[c0 + c]; xr[c0 + c] = v; s2 += v * v; }
+            for (int c = lane; c < n; c += 64) {
+                const float v = xr[c0 + c] + ld_f(x, c0 + c) * inv * w[c0 + c];
+                xr[c0 + c] = v; s2 += v * v;
+                if (plain) st_f(out, r * ldo + c0 + c, v);
+            }
             if (w2) {
                 const float inv2 = 1.0f / sqrtf(wave_sum(s2) / (float)n + eps);
                 for (int c = lane; c < n; c += 64) st_f(out, r * ldo + c0 + c, xr[c0 + c] * inv2 * w2[c0 + c]);   // (a lane re-reads what it wrote)
@@ -162,6 +166,91 @@ __device__ __forceinline__ void tile_product(const TileJob &j, int row0, int col
                 st_f(y, (int64_t)r * j.ldy + n, v);
             }
         }
+}
+
+// The same on the matrix cores for bfloat16 operands (K a multiple of 8, rows 16-byte aligned): v_mfma_f32_16x16x32_bf16, fragments straight from global
+// memory (a lane's 8 consecutive k of its row / column are one 16-byte load; nothing staged in LDS, no barrier).  WR = 4: the four waves take 16 rows each of
+// a 64 x 64 tile; WR = 1: they take 64 columns each of a 16 x 256 tile (few rows: decode-sized steps, experts with few tokens).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int WR>
+__device__ __forceinline__ void tile_product_mfma(const TileJob &j, int row0, int col0) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4;
+    const int rbase = row0 + (WR == 4 ? wave * 16 : 0), cbase = col0 + (WR == 4 ? 0 : wave * 64);
+    if (rbase >= j.rows || cbase >= j.N) return;
+    const bf16_t *w = (const bf16_t *)j.w;
+    const int r = rbase + lm;
+    const bool rok = r < j.rows;
+    const bf16_t *ap = (const bf16_t *)j.a; float rs = 1.f;
+    if (rok) {
+        if (j.src) { const int sidx = j.src[r]; ap += (int64_t)(sidx / j.src_div) * j.lda; rs = j.rscale[sidx]; }
+        else ap += (int64_t)r * j.lda;
+    }
+    const bf16_t *wp[4]; bool cok[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) { const int n = cbase + cb * 16 + lm; cok[cb] = n < j.N; wp[cb] = w + (int64_t)(cok[cb] ? n : 0) * j.ldw; }
+    f32x4 acc[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) acc[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const uint4 zero{0, 0, 0, 0};
+#pragma unroll 2
+    for (int k0 = 0; k0 < j.K; k0 += 32) {
+        const int k = k0 + lq * 8;
+        const bool kok = k < j.K;
+        uint4 av = (rok && kok) ? *reinterpret_cast<const uint4 *>(ap + k) : zero;
+        uint4 wv[4];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) wv[cb] = (cok[cb] && kok) ? *reinterpret_cast<const uint4 *>(wp[cb] + k) : zero;
+        if (j.src) {                                        // the scaled row is an operand: one rounding, as a stored copy would have
+            bf16_t *e = reinterpret_cast<bf16_t *>(&av);
+#pragma unroll
+            for (int y = 0; y < 8; ++y) st_f(e, y, ld_f(e, y) * rs);
+        }
+        const bf16x8 af = __builtin_bit_cast(bf16x8, av);
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, wv[cb]), acc[cb], 0, 0, 0);
+    }
+    bf16_t *y = (bf16_t *)j.y;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int rr = rbase + lq * 4 + i, n = cbase + cb * 16 + lm;
+            if (rr < j.rows && n < j.N) {
+                float v = acc[cb][i];
+                if (j.gate) v *= sigmoid_f(ld_f((const bf16_t *)j.gate, (int64_t)rr * j.ldg + n));
+                st_f(y, (int64_t)rr * j.ldy + n, v);
+            }
+        }
+}
+
+template <int WR>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinearArgs p) {
+    const int h = blockIdx.z;
+    TileJob j{};
+    j.a = (const bf16_t *)p.a + (int64_t)h * p.ha; j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)h * p.N * p.K; j.ldw = p.K;
+    j.y = (bf16_t *)p.y + (int64_t)h * p.hy; j.ldy = p.ldy; j.rows = p.T; j.K = p.K; j.N = p.N;
+    j.gate = p.gate ? (const void *)((const bf16_t *)p.gate + (int64_t)h * p.hg) : nullptr; j.ldg = p.ldg;
+    tile_product_mfma<WR>(j, blockIdx.y * (WR * 16), blockIdx.x * (WR == 4 ? 64 : 256));
+}
+
+template <int WR>
+__global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(GroupedLinearArgs p) {
+    constexpr int TR = WR * 16;
+    int tile = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < p.groups; ++e) {
+        lo = p.off[e]; hi = p.off[e + 1];
+        const int nt = (hi - lo + TR - 1) / TR;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (e == p.groups) return;
+    TileJob j{};
+    j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)e * p.N * p.K; j.ldw = p.K; j.y = (bf16_t *)p.y + (int64_t)lo * p.ldy; j.ldy = p.ldy;
+    j.rows = hi - lo; j.K = p.K; j.N = p.N;
+    if (p.src) { j.a = p.a; j.src = p.src + lo; j.rscale = p.rscale; j.src_div = p.src_div; }
+    else j.a = (const bf16_t *)p.a + (int64_t)lo * p.lda;
+    tile_product_mfma<WR>(j, tile * TR, blockIdx.x * (WR == 4 ? 64 : 256));
 }
 
 // y[t][h][n] = sum_k a[t][h][k] w[h][n][k]: blockIdx.z is the head
@@ -277,34 +366,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const OT *__restrict__
 }
 
 // ------------------------------------------------------------------------------------------------ end of a layer
-// Per row: (1) the token input: e = side_embed[id][ecol .. ecol + dim), g = gelu_tanh(Wg x) * e, y = Wp g, x += y / rms(y) * wn; (2) X_(i+1) = x goes to its
+// Per row: (1) the token input's last step: x += y / rms(y) * wn for the projected rows y (side_y); (2) X_(i+1) = x goes to its
 // place among the kept streams and x becomes sum_j mix[j] X_j over the nx kept streams (X_0 the embedding output ... X_(nx-1) this layer's); (3) with wnext the next layer's
 // first norm (in groups) of the new x goes to out.  Each part is optional (null pointers).  The row lives in LDS.
 template <class OT>
 __global__ __launch_bounds__(256) void layer_tail_kernel(LayerTailArgs p) {
-    extern __shared__ float sm[];                       // [W] x, [W] y, [dim] g
+    extern __shared__ float sm[];                       // [W] x, [W] y
     __shared__ float red[4];
     const int64_t t = blockIdx.x; const int W = p.W, lane = threadIdx.x & 63;
-    float *xs = sm, *ys = sm + W, *gs = ys + W;
+    float *xs = sm, *ys = sm + W;
     float *xr = p.x + t * W;
     for (int c = threadIdx.x; c < W; c += 256) xs[c] = xr[c];
     __syncthreads();
-    if (p.side_gate) {
-        const int64_t id = p.ids[t];
-        const OT *wg = (const OT *)p.side_gate, *wp = (const OT *)p.side_proj, *se = (const OT *)p.side_embed;
-        for (int d = threadIdx.x >> 6; d < p.dim; d += 4) {
-            float dot = 0.f;
-            for (int c = lane; c < W; c += 64) dot = fmaf(ld_f(wg, (int64_t)d * W + c), xs[c], dot);
-            dot = wave_sum(dot);
-            if (lane == 0) gs[d] = gelu_tanh_f(dot) * ld_f(se, id * p.side_ld + p.ecol + d);
-        }
-        __syncthreads();
+    if (p.side_y) {
+        const OT *sy = (const OT *)p.side_y + t * W;
         float ss = 0.f;
-        for (int c = threadIdx.x; c < W; c += 256) {
-            float y = 0.f;
-            for (int d = 0; d < p.dim; ++d) y = fmaf(ld_f(wp, (int64_t)c * p.dim + d), gs[d], y);
-            ys[c] = y; ss += y * y;
-        }
+        for (int c = threadIdx.x; c < W; c += 256) { const float y = ld_f(sy, c); ys[c] = y; ss += y * y; }
         ss = block_sum256(ss, red);
         const float inv = 1.0f / sqrtf(ss / (float)W + p.eps);
         for (int c = threadIdx.x; c < W; c += 256) xs[c] += ys[c] * inv * p.side_norm[c];
@@ -335,6 +412,16 @@ __global__ __launch_bounds__(256) void layer_tail_kernel(LayerTailArgs p) {
     }
 }
 
+// g[t][d] = gelu_tanh(z[t][d]) * E[ids[t]][ecol + d] (the token input between its two projections)
+template <class OT>
+__global__ __launch_bounds__(256) void side_gate_kernel(const OT *__restrict__ z, const int64_t *__restrict__ ids, const OT *__restrict__ E, int64_t lde, int ecol, int dim,
+                                                        int64_t n, OT *__restrict__ g) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int64_t t = idx / dim; const int d = (int)(idx - t * dim);
+    st_f(g, idx, gelu_tanh_f(ld_f(z, idx)) * ld_f(E, ids[t] * lde + ecol + d));
+}
+
 template <class ET>
 __global__ __launch_bounds__(256) void embed_keep_kernel(const ET *__restrict__ E, const int64_t *__restrict__ ids, int W, float *__restrict__ x, float *__restrict__ kept) {
     const int64_t t = blockIdx.x, id = ids[t];
@@ -361,17 +448,18 @@ int embed_keep(const void *E, bool bf16, const int64_t *ids, int64_t T, int64_t 
 int group_norm(const GroupNormArgs &a, bool bf16, hipStream_t s) {
     if (a.rows_n == 0) return 0;
     if (a.groups < 1 || a.W % a.groups) return nvr::fail(NVR_ERR_INVALID_ARG, "group_norm: %ld columns in %d groups", (long)a.W, a.groups);
+    if (a.out_plain && (a.w2 || !a.xres)) return nvr::fail(NVR_ERR_INVALID_ARG, "group_norm: a plain copy leaves only with the residual sum, instead of the next norm");
     const dim3 grid((unsigned)a.rows_n), blk(256);
     const int W = (int)a.W;
     if (a.xres) {                                        // operand-type rows joining the f32 stream
-        if (bf16) group_norm_kernel<bf16_t, bf16_t, true><<<grid, blk, 0, s>>>((const bf16_t *)a.in, a.ldi, nullptr, W, a.groups, a.eps, a.w, a.xres, a.w2, (bf16_t *)a.out, a.ldo);
-        else group_norm_kernel<float, float, true><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, nullptr, W, a.groups, a.eps, a.w, a.xres, a.w2, (float *)a.out, a.ldo);
+        if (bf16) group_norm_kernel<bf16_t, bf16_t, true><<<grid, blk, 0, s>>>((const bf16_t *)a.in, a.ldi, nullptr, W, a.groups, a.eps, a.w, a.xres, a.w2, a.out_plain ? 1 : 0, (bf16_t *)a.out, a.ldo);
+        else group_norm_kernel<float, float, true><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, nullptr, W, a.groups, a.eps, a.w, a.xres, a.w2, a.out_plain ? 1 : 0, (float *)a.out, a.ldo);
     } else if (a.in_f32) {
-        if (bf16) group_norm_kernel<float, bf16_t, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, (bf16_t *)a.out, a.ldo);
-        else group_norm_kernel<float, float, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, (float *)a.out, a.ldo);
+        if (bf16) group_norm_kernel<float, bf16_t, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, 0, (bf16_t *)a.out, a.ldo);
+        else group_norm_kernel<float, float, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, 0, (float *)a.out, a.ldo);
     } else {
-        if (bf16) group_norm_kernel<bf16_t, bf16_t, false><<<grid, blk, 0, s>>>((const bf16_t *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, (bf16_t *)a.out, a.ldo);
-        else group_norm_kernel<float, float, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, (float *)a.out, a.ldo);
+        if (bf16) group_norm_kernel<bf16_t, bf16_t, false><<<grid, blk, 0, s>>>((const bf16_t *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, 0, (bf16_t *)a.out, a.ldo);
+        else group_norm_kernel<float, float, false><<<grid, blk, 0, s>>>((const float *)a.in, a.ldi, a.rows, W, a.groups, a.eps, a.w, nullptr, nullptr, 0, (float *)a.out, a.ldo);
     }
     return launched("group_norm");
 }
@@ -394,8 +482,15 @@ int rotate_heads(const void *q, int64_t ldq, int64_t qstride, int64_t qcol, cons
     return launched("rotate_heads");
 }
 
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
 int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.T == 0 || a.N == 0 || a.H == 0) return 0;
+    if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && a.ha % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
+        if (a.T <= 16) head_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)((a.T + 15) / 16), (unsigned)a.H), dim3(256), 0, s>>>(a);
+        else head_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)((a.T + 63) / 64), (unsigned)a.H), dim3(256), 0, s>>>(a);
+        return launched("head_linear");
+    }
     const dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((a.T + 63) / 64), (unsigned)a.H);
     if (bf16) head_linear_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a);
     else head_linear_kernel<float><<<grid, dim3(256), 0, s>>>(a);
@@ -404,6 +499,11 @@ int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s) {
 
 int grouped_linear(const GroupedLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.max_rows == 0 || a.N == 0 || a.groups == 0) return 0;
+    if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
+        if (a.max_rows <= 16 * a.groups) grouped_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.max_rows / 16 + a.groups)), dim3(256), 0, s>>>(a);
+        else grouped_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)(a.max_rows / 64 + a.groups)), dim3(256), 0, s>>>(a);
+        return launched("grouped_linear");
+    }
     const dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)(a.max_rows / 64 + a.groups));
     if (bf16) grouped_linear_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(a);
     else grouped_linear_kernel<float><<<grid, dim3(256), 0, s>>>(a);
@@ -444,9 +544,17 @@ int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, 
     return launched("moe_combine");
 }
 
+int side_gate(const void *z, const int64_t *ids, const void *E, int64_t lde, int64_t ecol, int64_t dim, int64_t T, void *g, bool bf16, hipStream_t s) {
+    if (T * dim == 0) return 0;
+    const dim3 grid((unsigned)((T * dim + 255) / 256));
+    if (bf16) side_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((const bf16_t *)z, ids, (const bf16_t *)E, lde, (int)ecol, (int)dim, T * dim, (bf16_t *)g);
+    else side_gate_kernel<float><<<grid, dim3(256), 0, s>>>((const float *)z, ids, (const float *)E, lde, (int)ecol, (int)dim, T * dim, (float *)g);
+    return launched("side_gate");
+}
+
 int layer_tail(const LayerTailArgs &a, bool bf16, hipStream_t s) {
     if (a.T == 0) return 0;
-    const size_t lds = ((size_t)2 * a.W + (size_t)std::max(a.dim, 1)) * 4;
+    const size_t lds = (size_t)2 * a.W * 4;
     if (lds > kMaxLds) return nvr::fail(NVR_ERR_UNSUPPORTED, "layer_tail: rows of %d numbers do not fit LDS", a.W);
     if (a.wnext && (a.groups < 1 || a.W % a.groups)) return nvr::fail(NVR_ERR_INVALID_ARG, "layer_tail: %d columns in %d groups", a.W, a.groups);
     if (bf16) layer_tail_kernel<bf16_t><<<dim3((unsigned)a.T), dim3(256), lds, s>>>(a);

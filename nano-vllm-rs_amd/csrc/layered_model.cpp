@@ -485,6 +485,11 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
             for (int64_t j = 0; j < R / 2; ++j) f[(size_t)j] = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
             RC(own(&w.rfreq, f.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.rfreq, f.data(), f.size() * 4, hipMemcpyHostToDevice));
             max_qabs = std::max(max_qabs, L.heads * (L.kv_rank + R)); max_ctx = std::max(max_ctx, L.heads * L.kv_rank);
+            // the matrix-core attention takes up to 16 query heads per key/value row: the heads go in equal shares of the largest divisor of H up to 16
+            int64_t g = std::min<int64_t>(L.heads, 16);
+            while (L.heads % g) --g;
+            w.head_share = g;
+            if (std::find(attn_groups.begin(), attn_groups.end(), g) == attn_groups.end()) attn_groups.push_back(g);
         } else if (L.mixer == LayeredSpec::GLA) {
             w.qcol = 0; w.kcol = hd; w.vcol = 2 * hd; w.gcol = 2 * hd + hv; w.nmix = 2 * hd + 2 * hv;
             RC(own(&w.a2b, (size_t)hd * 4)); RC(own(&w.hnorm, (size_t)L.vdim * 4));
@@ -539,6 +544,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
     RC(named((void **)&ret_o, (size_t)(MT * max_hv * 4))); RC(own(&az, (size_t)(MT * max_hd * esz)));
     RC(named(&gu, (size_t)(MT * max_ff * esz))); RC(own(&act, (size_t)(MT * max_ff * esz))); RC(own(&shared_y, (size_t)(MT * W * esz)));
     RC(own(&e_gu, (size_t)(MT * max_e2f * esz))); RC(own(&e_act, (size_t)(MT * max_ef * esz))); RC(own(&e_y, (size_t)(MT * max_rows_e * W * esz)));
+    RC(own(&side_z, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz))); RC(own(&side_g, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz)));
     RC(own(&moe_i, (size_t)((3 * MT * std::max<int64_t>(max_rows_e, 1) + 1024 + 8) * 4))); RC(own(&moe_score, (size_t)(MT * std::max<int64_t>(max_rows_e, 1) * 4)));
     return NVR_OK;
 }
@@ -674,7 +680,20 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
             kl::SinkAttnArgs a{};
             a.q = qabs; a.ldq = L.heads * Dq; a.kc = st.kc; a.vc = st.kc; a.vld = Dq; a.H = (int32_t)L.heads; a.G = 1; a.D = (int32_t)Dq; a.Dv = (int32_t)rank;
             a.scale = (float)L.scale; a.out = ctx; a.ldo = L.heads * rank;
-            RC(kl::sink_attention(a, b, bf16, s));
+            kl::SinkAttnArgs a1s = a; a1s.H = (int32_t)w.head_share;
+            if (kl::sink_attention_tiled_ok(a1s, bf16, (int)r.block_size)) {
+                const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), w.head_share) - attn_groups.begin());
+                const int64_t wgs = (int64_t)p.n_tiles[gi];
+                int64_t nsplit = 1;
+                if (wgs * (L.heads / w.head_share) < r.num_cus && p.max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / (wgs * (L.heads / w.head_share)), (p.max_ctx + 255) / 256, 16}));
+                const size_t share_ws = attn_ws_bytes / (size_t)(L.heads / w.head_share);
+                for (int64_t h0 = 0; h0 < L.heads; h0 += w.head_share) {       // one launch per share of the heads, all on the same cached rows
+                    kl::SinkAttnArgs as = a1s;
+                    as.q = (const char *)qabs + (size_t)(h0 * Dq * esz); as.out = (char *)ctx + (size_t)(h0 * rank * esz);
+                    RC(kl::sink_attention_tiled(as, b, (const kl::AttnTile *)(in_dev + p.o_tiles[gi]), p.n_tiles[gi], (int)nsplit, (char *)attn_ws + (size_t)(h0 / w.head_share) * share_ws, share_ws, s));
+                }
+            } else
+                RC(kl::sink_attention(a, b, bf16, s));
             // the value expansion of the attended latent, and the output gate
             kl::HeadLinearArgs hu{}; hu.a = ctx; hu.lda = L.heads * rank; hu.ha = rank; hu.w = w.uv; hu.y = cat; hu.ldy = hv; hu.hy = L.vdim;
             hu.T = (int32_t)T; hu.H = (int32_t)L.heads; hu.K = (int32_t)rank; hu.N = (int32_t)L.vdim;
@@ -695,6 +714,7 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
         {   // the mixer's output joins the stream; the feed-forward's input leaves in the same pass
             kl::GroupNormArgs n{}; n.in = tmp; n.ldi = W; n.rows_n = T; n.W = W; n.groups = groups; n.eps = eps; n.w = w.n1b; n.xres = x;
             if (L.has_mlp) { n.w2 = w.n2; n.out = a2; n.ldo = W; }
+            else if (spec.side_dim && bf16) { n.out_plain = true; n.out = a2; n.ldo = W; }       // (the token input's projection reads the stream in the operand type)
             RC(kl::group_norm(n, bf16, s));
         }
         if (L.ff_kind == LayeredSpec::FF_POLY) {
@@ -720,10 +740,16 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
         }
         if (L.has_mlp) {
             kl::GroupNormArgs n{}; n.in = tmp; n.ldi = W; n.rows_n = T; n.W = W; n.groups = groups; n.eps = eps; n.w = w.n2b; n.xres = x;
+            if (spec.side_dim && bf16) { n.out_plain = true; n.out = a2; n.ldo = W; }
             RC(kl::group_norm(n, bf16, s));
         }
-        kl::LayerTailArgs t{}; t.x = x; t.T = (int32_t)T; t.W = (int32_t)W; t.eps = eps; t.ids = b.ids;
-        if (spec.side_dim) { t.side_embed = side_embed; t.side_ld = nL * spec.side_dim; t.ecol = (int32_t)(i * spec.side_dim); t.dim = (int32_t)spec.side_dim; t.side_gate = w.sgate; t.side_proj = w.sproj; t.side_norm = w.snorm; }
+        kl::LayerTailArgs t{}; t.x = x; t.T = (int32_t)T; t.W = (int32_t)W; t.eps = eps;
+        if (spec.side_dim) {                                // the token input: two products around the gate, its norm at the end of the layer
+            RC(gemm(r, bf16 ? a2 : (void *)x, W, w.sgate, T, W, spec.side_dim, side_z));
+            RC(kl::side_gate(side_z, b.ids, side_embed, nL * spec.side_dim, i * spec.side_dim, spec.side_dim, T, side_g, bf16, s));
+            RC(gemm(r, side_g, spec.side_dim, w.sproj, T, spec.side_dim, W, tmp));
+            t.side_y = tmp; t.side_norm = w.snorm;
+        }
         t.kept = kept; t.kept_rows = MT; t.nx = (int32_t)(i + 2); t.mix = w.dwa;
         if (i + 1 < nL) { t.wnext = lw[(size_t)(i + 1)].n1; t.groups = groups; t.out = a1; }
         RC(kl::layer_tail(t, bf16, s));

@@ -72,6 +72,7 @@ public:
         int64_t qcol = 0, kcol = 0, vcol = 0, gcol = 0;
         // sequential layout
         float *n1 = nullptr, *n1b = nullptr, *n2 = nullptr, *n2b = nullptr;         // [W] each
+        int64_t head_share = 0;                             // latent attention on the matrix cores: query heads per launch
         int64_t dcol = 0;                                   // latent attention: column of the (queries' latent,) cached row's source in the mix projection
         void *uq = nullptr, *ukt = nullptr, *uv = nullptr, *wo = nullptr;            // [H (D + R)][q_rank]; [H][kv_rank][D] (Wuk per head, transposed); [H][Dv][kv_rank]; [W][H Dv]
         float *dqn = nullptr, *dkvn = nullptr, *rfreq = nullptr;                     // latent norms' weights, rotation frequencies [rot_dim / 2]
@@ -88,7 +89,7 @@ public:
     float *wfinal = nullptr; void *side_embed = nullptr;                    // [W]; [vocab][layers * side_dim]
     float *kept = nullptr;                                                  // the embedding output and every layer's output: [layers + 1][max tokens][W] f32
     void *qlat = nullptr, *q2 = nullptr, *qabs = nullptr, *ctx = nullptr, *alow = nullptr, *az = nullptr, *act = nullptr, *shared_y = nullptr;
-    int64_t alow_cap = 0;
+    int64_t alow_cap = 0; void *side_z = nullptr, *side_g = nullptr;
     void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
     // activations

@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of a Rugudra-design model beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
+"""Prefill and decode throughput of the layer-list designs (Rugudra, Pusunex) beside the dense Qwen3 graph at equal sizes (bench.py --layered-compare).
 
 Random weights, layer shapes that resemble a real model's; both models go through the same engine (scheduler, block manager, runner step).
 Per size one JSON object: tokens/s of one prefill step over BATCH prompts of PROMPT tokens and of the decode steps that follow, for both."""
@@ -62,6 +62,67 @@ def random_weights(cfg, seed=0):
     return out
 
 
+def pusunex_config(s):
+    """Layers in turn: latent attention with a dense feed-forward, latent attention on the first layer's cached rows with experts, gated linear attention
+    with experts, latent attention with latent queries and a rotated key part with experts.  The experts' sizes add up to the dense feed-forward's:
+    8 experts of ff / 4, two chosen per token, and a shared one of ff / 2."""
+    H, D, W = s["heads"], s["dim"], s["width"]
+    experts = {"kind": "moe", "expert": {"ff": s["ff"] // 4}, "router": {"experts": 8, "top": 2}, "shared": {"ff": s["ff"] // 2}}
+    layers = []
+    for i in range(s["layers"]):
+        k = i % 4
+        if k == 0:
+            layers.append({"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": 256, "scale": D ** -0.5}, "mlp": {"kind": "dense", "ff": s["ff"]}})
+        elif k == 1:
+            layers.append({"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": 256, "kv_from": i - 1, "scale": D ** -0.5}, "mlp": experts})
+        elif k == 2:
+            layers.append({"type": "gla", "mixer": {"heads": H, "dim": D, "vdim": D, "tau": 16.0}, "mlp": experts})
+        else:
+            layers.append({"type": "latent_attention_2", "mixer": {"heads": H, "dim": D - 64, "rot_dim": 64, "vdim": D, "kv_rank": 192, "q_rank": W // 2,
+                                                                    "rot": {"dims": 64, "base": 10000.0}, "scale": D ** -0.5}, "mlp": experts})
+    return {"architecture": "Pusunex", "vocab": s["vocab"], "width": W, "norm": {"eps": 1e-6, "groups": 4}, "token_side": {"dim": 64}, "layers": layers}
+
+
+def pusunex_weights(cfg, seed=0):
+    rng = np.random.default_rng(seed)
+    W, V, nL, side = cfg["width"], cfg["vocab"], len(cfg["layers"]), cfg["token_side"]["dim"]
+
+    def lin(o, i, g=1.0):
+        return (rng.standard_normal((o, i), dtype=np.float32) * (g / np.sqrt(i))).astype(np.float32)
+
+    def gains(n):
+        return (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    out = {"embed": rng.standard_normal((V, W), dtype=np.float32), "head": lin(V, W), "final.norm": gains(W), "side.embed": rng.standard_normal((V, nL * side), dtype=np.float32)}
+    for i, L in enumerate(cfg["layers"]):
+        m, p = L["mixer"], "l%d." % i
+        H, D, Dv = m["heads"], m["dim"], m["vdim"]
+        out[p + "norm1"], out[p + "norm1b"], out[p + "norm2"], out[p + "norm2b"] = gains(W), gains(W), gains(W), gains(W)
+        if L["type"] == "gla":
+            out[p + "mix.q"], out[p + "mix.k"], out[p + "mix.v"], out[p + "mix.g"] = lin(H * D, W), lin(H * D, W), lin(H * Dv, W), lin(H * Dv, W)
+            out[p + "mix.norm"], out[p + "mix.a1"], out[p + "mix.a2"] = gains(Dv), lin(32, W), lin(H * D, 32)
+            out[p + "mix.a2.b"] = (3.0 + rng.standard_normal(H * D)).astype(np.float32)
+        else:
+            rank, R = m["kv_rank"], m.get("rot_dim", 0)
+            if "q_rank" in m:
+                out[p + "mix.dq"], out[p + "mix.dq.norm"], out[p + "mix.uq"] = lin(m["q_rank"], W), gains(m["q_rank"]), lin(H * (D + R), m["q_rank"])
+            else:
+                out[p + "mix.q"], out[p + "mix.g"] = lin(H * D, W), lin(H * Dv, W)
+            if m.get("kv_from") is None:
+                out[p + "mix.dkv"], out[p + "mix.dkv.norm"] = lin(rank + R, W), gains(rank)
+            out[p + "mix.uk"], out[p + "mix.uv"] = lin(H * D, rank), lin(H * Dv, rank)
+        out[p + "mix.o"] = lin(W, H * Dv)
+        mlp = L["mlp"]
+        if mlp["kind"] == "dense":
+            out[p + "mlp.up"], out[p + "mlp.down"], out[p + "mlp.act"] = lin(mlp["ff"], W), lin(W, mlp["ff"]), np.array([0.7, 0.4, -0.3, 0.1], np.float32)
+        else:
+            out[p + "mlp.router"] = lin(mlp["router"]["experts"], W, 2.0)
+            for n, f in [("e%d" % e, mlp["expert"]["ff"]) for e in range(mlp["router"]["experts"])] + [("shared", mlp["shared"]["ff"])]:
+                out[p + "mlp.%s.gate" % n], out[p + "mlp.%s.up" % n], out[p + "mlp.%s.down" % n] = lin(f, W), lin(f, W), lin(W, f)
+        out[p + "side.gate"], out[p + "side.proj"], out[p + "side.norm"] = lin(side, W), lin(W, side), (0.3 * gains(W)).astype(np.float32)
+        out[p + "dwa"] = np.concatenate([0.1 * rng.standard_normal(i + 1), [1.0]]).astype(np.float32)
+    return out
+
+
 def _run(nvr, engine, vocab, batch, prompt, steps, warmup):
     sp = nvr.SamplingParams(temperature=0.0, max_tokens=steps + warmup + 1, ignore_eos=True)
     for i in range(batch):
@@ -99,6 +160,14 @@ def compare(nvr, sizes=("w1024", "w2048"), batch=16, prompt=1024, steps=32, warm
                 eng.model_runner.load_tensor(k, np.asarray(v))
             _run(nvr, eng, s["vocab"], 2, 64, 2, 1)                       # first launches
             line["rugudra"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
+            del eng
+        if "pusunex" in which:
+            cfg = pusunex_config(s)
+            eng = nvr.LLMEngine(nvr.Config(**ecfg), nvr.ModelSpec(cfg))
+            for k, v in pusunex_weights(cfg).items():
+                eng.model_runner.load_tensor(k, np.asarray(v))
+            _run(nvr, eng, s["vocab"], 2, 64, 2, 1)
+            line["pusunex"] = _run(nvr, eng, s["vocab"], batch, prompt, steps, warmup)
             del eng
         if "qwen3" in which:
             m = nvr.ModelConfig(vocab_size=s["vocab"], hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=s["layers"], num_attention_heads=s["heads"],
