@@ -574,6 +574,23 @@ __global__ __launch_bounds__(256) void retention_block_kernel(RetentionArgs a, B
                     ks[i * D + d0 + y] = (ku * cs - kv * sn) * a.kscale; ks[i * D + half + d0 + y] = (kv * cs + ku * sn) * a.kscale;
                 }
             }
+        } else if (GATED && sizeof(PT) == 2 && a.rot_dims == 0 && (D & 7) == 0 && (a.ld & 7) == 0 && ((a.qcol | a.kcol | a.ldz) & 7) == 0 && (((uintptr_t)a.proj | (uintptr_t)a.az) & 15) == 0) {
+            // gated, 16-bit rows: a thread takes 8 consecutive channels of one token as 16-byte loads; the decay (1 + e^-z)^(-1/tau) through the hardware's
+            // base-2 exponential and logarithm (z -> -inf gives 0, no overflow on the way)
+            const int cpt = D >> 3;
+            for (int idx = threadIdx.x; idx < nb * cpt; idx += 256) {
+                const int i = idx / cpt, d0 = (idx - i * cpt) << 3;
+                const bf16_t *pr = (const bf16_t *)a.proj + (int64_t)(r0 + i0 + i) * a.ld;
+                const uint4 qv = *reinterpret_cast<const uint4 *>(pr + a.qcol + (int64_t)h * D + d0), kv = *reinterpret_cast<const uint4 *>(pr + a.kcol + (int64_t)h * D + d0);
+                const uint4 zv = *reinterpret_cast<const uint4 *>((const bf16_t *)a.az + (int64_t)(r0 + i0 + i) * a.ldz + (int64_t)h * D + d0);
+                const bf16_t *qe = reinterpret_cast<const bf16_t *>(&qv), *ke = reinterpret_cast<const bf16_t *>(&kv), *ze = reinterpret_cast<const bf16_t *>(&zv);
+                const float *bp = a.abias + (int64_t)h * D + d0;
+#pragma unroll
+                for (int y = 0; y < 8; ++y) {
+                    qs[i * D + d0 + y] = ld_f(qe, y) * a.qscale; ks[i * D + d0 + y] = ld_f(ke, y) * a.kscale;
+                    as[i * D + d0 + y] = exp2f(-a.inv_tau * __log2f(1.0f + exp2f(-kLog2e * (ld_f(ze, y) + bp[y]))));
+                }
+            }
         } else
         for (int idx = threadIdx.x; idx < nb * D; idx += 256) {
             const int i = dsh >= 0 ? idx >> dsh : idx / D, d = idx - i * D;

@@ -224,6 +224,112 @@ __device__ __forceinline__ void tile_product_mfma(const TileJob &j, int row0, in
         }
 }
 
+// Many rows: a 128 x 128 tile per workgroup, K in steps of 32 through LDS (the next step's 16-byte pieces are requested before the current step's
+// arithmetic); the four waves own 64 x 64 quarters, 16 MFMAs per step from 8 fragments.
+__device__ __forceinline__ void tile_product_mfma128(const TileJob &j, int row0, int col0, bf16_t *As, bf16_t *Ws) {
+    constexpr int LD = 40;                                  // 32 + 8 elements: rows stay 16-byte aligned and spread over the banks
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4, wr = wave >> 1, wc = wave & 1;
+    const int lrow = threadIdx.x >> 2, lch = threadIdx.x & 3;
+    const bf16_t *ap[2], *wp[2]; bool aok[2], wok[2]; float rs[2] = {1.f, 1.f};
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int r = row0 + lrow + 64 * q, n = col0 + lrow + 64 * q;
+        aok[q] = r < j.rows; wok[q] = n < j.N;
+        ap[q] = (const bf16_t *)j.a; wp[q] = (const bf16_t *)j.w + (int64_t)(wok[q] ? n : 0) * j.ldw;
+        if (aok[q]) {
+            if (j.src) { const int sidx = j.src[r]; ap[q] += (int64_t)(sidx / j.src_div) * j.lda; rs[q] = j.rscale[sidx]; }
+            else ap[q] += (int64_t)r * j.lda;
+        }
+    }
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[i][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const uint4 zero{0, 0, 0, 0};
+    uint4 ra[2], rw[2];
+    auto fetch = [&](int k0) {
+        const int k = k0 + lch * 8;
+        const bool kok = k < j.K;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            ra[q] = (aok[q] && kok) ? *reinterpret_cast<const uint4 *>(ap[q] + k) : zero;
+            rw[q] = (wok[q] && kok) ? *reinterpret_cast<const uint4 *>(wp[q] + k) : zero;
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < j.K; k0 += 32) {
+        if (j.src) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                bf16_t *e = reinterpret_cast<bf16_t *>(&ra[q]);
+#pragma unroll
+                for (int y = 0; y < 8; ++y) st_f(e, y, ld_f(e, y) * rs[q]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            *reinterpret_cast<uint4 *>(As + (lrow + 64 * q) * LD + lch * 8) = ra[q];
+            *reinterpret_cast<uint4 *>(Ws + (lrow + 64 * q) * LD + lch * 8) = rw[q];
+        }
+        __syncthreads();
+        if (k0 + 32 < j.K) fetch(k0 + 32);
+        bf16x8 af[4], wf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            af[i] = *reinterpret_cast<const bf16x8 *>(As + (wr * 64 + i * 16 + lm) * LD + lq * 8);
+            wf[i] = *reinterpret_cast<const bf16x8 *>(Ws + (wc * 64 + i * 16 + lm) * LD + lq * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[c], acc[i][c], 0, 0, 0);
+    }
+    bf16_t *y = (bf16_t *)j.y;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int rr = row0 + wr * 64 + i * 16 + lq * 4 + e, n = col0 + wc * 64 + c * 16 + lm;
+                if (rr < j.rows && n < j.N) {
+                    float v = acc[i][c][e];
+                    if (j.gate) v *= sigmoid_f(ld_f((const bf16_t *)j.gate, (int64_t)rr * j.ldg + n));
+                    st_f(y, (int64_t)rr * j.ldy + n, v);
+                }
+            }
+}
+
+__global__ __launch_bounds__(256) void head_linear_mfma128_kernel(HeadLinearArgs p) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 40], Ws[128 * 40];
+    const int h = blockIdx.z;
+    TileJob j{};
+    j.a = (const bf16_t *)p.a + (int64_t)h * p.ha; j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)h * p.N * p.K; j.ldw = p.K;
+    j.y = (bf16_t *)p.y + (int64_t)h * p.hy; j.ldy = p.ldy; j.rows = p.T; j.K = p.K; j.N = p.N;
+    j.gate = p.gate ? (const void *)((const bf16_t *)p.gate + (int64_t)h * p.hg) : nullptr; j.ldg = p.ldg;
+    tile_product_mfma128(j, blockIdx.y * 128, blockIdx.x * 128, As, Ws);
+}
+
+__global__ __launch_bounds__(256) void grouped_linear_mfma128_kernel(GroupedLinearArgs p) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 40], Ws[128 * 40];
+    int tile = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < p.groups; ++e) {
+        lo = p.off[e]; hi = p.off[e + 1];
+        const int nt = (hi - lo + 127) >> 7;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (e == p.groups) return;                              // (every thread of the workgroup leaves: no barrier is left waiting)
+    TileJob j{};
+    j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)e * p.N * p.K; j.ldw = p.K; j.y = (bf16_t *)p.y + (int64_t)lo * p.ldy; j.ldy = p.ldy;
+    j.rows = hi - lo; j.K = p.K; j.N = p.N;
+    if (p.src) { j.a = p.a; j.src = p.src + lo; j.rscale = p.rscale; j.src_div = p.src_div; }
+    else j.a = (const bf16_t *)p.a + (int64_t)lo * p.lda;
+    tile_product_mfma128(j, tile * 128, blockIdx.x * 128, As, Ws);
+}
+
 template <int WR>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinearArgs p) {
     const int h = blockIdx.z;
@@ -487,7 +593,8 @@ static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.T == 0 || a.N == 0 || a.H == 0) return 0;
     if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && a.ha % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
-        if (a.T <= 16) head_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)((a.T + 15) / 16), (unsigned)a.H), dim3(256), 0, s>>>(a);
+        if (a.T >= 128) head_linear_mfma128_kernel<<<dim3((unsigned)((a.N + 127) / 128), (unsigned)((a.T + 127) / 128), (unsigned)a.H), dim3(256), 0, s>>>(a);
+        else if (a.T <= 16) head_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)((a.T + 15) / 16), (unsigned)a.H), dim3(256), 0, s>>>(a);
         else head_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)((a.T + 63) / 64), (unsigned)a.H), dim3(256), 0, s>>>(a);
         return launched("head_linear");
     }
@@ -500,7 +607,8 @@ int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s) {
 int grouped_linear(const GroupedLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.max_rows == 0 || a.N == 0 || a.groups == 0) return 0;
     if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
-        if (a.max_rows <= 16 * a.groups) grouped_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.max_rows / 16 + a.groups)), dim3(256), 0, s>>>(a);
+        if (a.max_rows >= 96 * a.groups) grouped_linear_mfma128_kernel<<<dim3((unsigned)((a.N + 127) / 128), (unsigned)(a.max_rows / 128 + a.groups)), dim3(256), 0, s>>>(a);
+        else if (a.max_rows <= 16 * a.groups) grouped_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.max_rows / 16 + a.groups)), dim3(256), 0, s>>>(a);
         else grouped_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)(a.max_rows / 64 + a.groups)), dim3(256), 0, s>>>(a);
         return launched("grouped_linear");
     }

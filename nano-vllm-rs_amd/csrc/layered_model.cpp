@@ -685,7 +685,7 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
                 const size_t gi = (size_t)(std::find(attn_groups.begin(), attn_groups.end(), w.head_share) - attn_groups.begin());
                 const int64_t wgs = (int64_t)p.n_tiles[gi];
                 int64_t nsplit = 1;
-                if (wgs * (L.heads / w.head_share) < r.num_cus && p.max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / (wgs * (L.heads / w.head_share)), (p.max_ctx + 255) / 256, 16}));
+                if (wgs * (L.heads / w.head_share) < r.num_cus && p.max_ctx >= 512) nsplit = std::max<int64_t>(1, std::min<int64_t>({(2 * r.num_cus) / (wgs * (L.heads / w.head_share)), (p.max_ctx + 127) / 128, 16}));
                 const size_t share_ws = attn_ws_bytes / (size_t)(L.heads / w.head_share);
                 for (int64_t h0 = 0; h0 < L.heads; h0 += w.head_share) {       // one launch per share of the heads, all on the same cached rows
                     kl::SinkAttnArgs as = a1s;

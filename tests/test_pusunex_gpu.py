@@ -57,6 +57,18 @@ def test_mechanism_alone(name, dtype):
     check(d.run_alone(toks), expected_logits(cfg, w, toks), dtype, name)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_products_per_head_and_per_expert_with_many_rows(dtype):
+    """A prompt long enough for the large tiles of the per-head and per-expert products (128 rows and more per head, about a hundred per expert), in one
+    step and in two uneven ones."""
+    cfg = make_config([latent_layer(heads=2, dim=32, vdim=24, kv_rank=40, mlp=moe(3, 2, 40, 24)), latent2_layer(mlp=moe(2, 1, 24, 0))], side=4)
+    w = make_weights(cfg, seed=21)
+    toks = settled_tokens(cfg, w, 300, 22)
+    want = expected_logits(cfg, w, toks)
+    check(Driver(cfg, w, dtype, page=16, pages=40, max_tokens=512).run_alone(toks), want, dtype, "one step")
+    check(Driver(cfg, w, dtype, page=16, pages=40, max_tokens=512).run_alone(toks, cuts=[171, 129]), want, dtype, "two steps")
+
+
 def test_each_part_changes_the_result():
     """A part that is left out must show: with the output gate's, the decay's, the token input's or the depth average's weights changed the restatement's
     logits move by far more than the tolerance, and the engine follows each variant."""
