@@ -110,9 +110,12 @@ struct GroupNormArgs {
 int group_norm(const GroupNormArgs &a, bool bf16, hipStream_t s);
 
 // Latent attention caches ONE row per token: `rank` numbers of the latent (proj columns col ..., divided by their root mean square, times w) and `rot` numbers of a
-// key part shared by the heads, rotated in pairs (2i, 2i+1) by position * freq[i].  pages: [blocks][block_size][rank + rot] of the operand type.
-int latent_store(const void *proj, int64_t ld, int64_t col, const Batch &b, int64_t rank, int64_t rot, float eps, const float *w, const float *freq, void *pages, bool bf16,
-                 hipStream_t s);
+// key part shared by the heads, rotated in pairs (2i, 2i+1) by position * freq[i].  pages: [blocks][block_size][rank + rot] of the operand type; rows (may be null):
+// the same rows in step order, [T][rank + rot].
+int latent_store(const void *proj, int64_t ld, int64_t col, const Batch &b, int64_t rank, int64_t rot, float eps, const float *w, const float *freq, void *pages, void *rows,
+                 bool bf16, hipStream_t s);
+// y[t][c] *= sigmoid(g[t][c]) (c < N; rows of y / g with strides ldy / ldg)
+int sigmoid_gate(void *y, int64_t ldy, const void *g, int64_t ldg, int64_t T, int64_t N, bool bf16, hipStream_t s);
 // The rotated part of the queries: q[t][h * qstride + qcol ...] (rot numbers, pairs (2i, 2i+1)) -> out[t][h * ostride + ocol ...]
 int rotate_heads(const void *q, int64_t ldq, int64_t qstride, int64_t qcol, const Batch &b, int64_t H, int64_t rot, const float *freq, void *out, int64_t ldo, int64_t ostride,
                  int64_t ocol, bool bf16, hipStream_t s);

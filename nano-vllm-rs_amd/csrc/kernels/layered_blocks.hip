@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void group_norm_kernel(const IT *__restrict__ 
 // divided by its root mean square times w, and the key part with coordinate pairs (2i, 2i+1) turned by position * freq[i].
 template <class CT>
 __global__ __launch_bounds__(64) void latent_store_kernel(const CT *__restrict__ proj, int64_t ld, int64_t col, Batch b, int rank, int rot, float eps,
-                                                          const float *__restrict__ w, const float *__restrict__ freq, CT *__restrict__ pages) {
+                                                          const float *__restrict__ w, const float *__restrict__ freq, CT *__restrict__ pages, CT *__restrict__ rows) {
     const int t = blockIdx.x, sq = b.row_seq[t], lane = threadIdx.x;
     const int p = b.start[sq] + (t - b.cu[sq]);
     const int blk = b.block_tables[(int64_t)sq * b.max_blocks + p / b.block_size];
@@ -91,11 +91,13 @@ __global__ __launch_bounds__(64) void latent_store_kernel(const CT *__restrict__
     float ss = 0.f;
     for (int c = lane; c < rank; c += 64) { const float v = ld_f(src, c); ss += v * v; }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)rank + eps);
-    for (int c = lane; c < rank; c += 64) st_f(dst, c, ld_f(src, c) * inv * w[c]);
+    CT *dst2 = rows ? rows + (int64_t)t * (rank + rot) : nullptr;      // the same row once more, in step order
+    for (int c = lane; c < rank; c += 64) { const float v = ld_f(src, c) * inv * w[c]; st_f(dst, c, v); if (dst2) st_f(dst2, c, v); }
     for (int i = lane; i < rot / 2; i += 64) {
         const float ang = (float)p * freq[i], cs = cosf(ang), sn = sinf(ang);
         const float u = ld_f(src, rank + 2 * i), v = ld_f(src, rank + 2 * i + 1);
         st_f(dst, rank + 2 * i, u * cs - v * sn); st_f(dst, rank + 2 * i + 1, v * cs + u * sn);
+        if (dst2) { st_f(dst2, rank + 2 * i, u * cs - v * sn); st_f(dst2, rank + 2 * i + 1, v * cs + u * sn); }
     }
 }
 
@@ -224,16 +226,16 @@ __device__ __forceinline__ void tile_product_mfma(const TileJob &j, int row0, in
         }
 }
 
-// Many rows: a 128 x 128 tile per workgroup, K in steps of 32 through LDS (the next step's 16-byte pieces are requested before the current step's
-// arithmetic); the four waves own 64 x 64 quarters, 16 MFMAs per step from 8 fragments.
+// Many rows: a 128 x 128 tile per workgroup, K in steps of 64 through LDS (the next step's 16-byte pieces are requested before the current step's
+// arithmetic); the four waves own 64 x 64 quarters, 32 MFMAs per step.
 __device__ __forceinline__ void tile_product_mfma128(const TileJob &j, int row0, int col0, bf16_t *As, bf16_t *Ws) {
-    constexpr int LD = 40;                                  // 32 + 8 elements: rows stay 16-byte aligned and spread over the banks
+    constexpr int KS = 64, LD = KS + 8;                     // rows stay 16-byte aligned and spread over the banks
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4, wr = wave >> 1, wc = wave & 1;
-    const int lrow = threadIdx.x >> 2, lch = threadIdx.x & 3;
-    const bf16_t *ap[2], *wp[2]; bool aok[2], wok[2]; float rs[2] = {1.f, 1.f};
+    const int lrow = threadIdx.x >> 3, lch = threadIdx.x & 7;
+    const bf16_t *ap[4], *wp[4]; bool aok[4], wok[4]; float rs[4] = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int r = row0 + lrow + 64 * q, n = col0 + lrow + 64 * q;
+    for (int q = 0; q < 4; ++q) {
+        const int r = row0 + lrow + 32 * q, n = col0 + lrow + 32 * q;
         aok[q] = r < j.rows; wok[q] = n < j.N;
         ap[q] = (const bf16_t *)j.a; wp[q] = (const bf16_t *)j.w + (int64_t)(wok[q] ? n : 0) * j.ldw;
         if (aok[q]) {
@@ -247,21 +249,21 @@ __device__ __forceinline__ void tile_product_mfma128(const TileJob &j, int row0,
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[i][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     const uint4 zero{0, 0, 0, 0};
-    uint4 ra[2], rw[2];
+    uint4 ra[4], rw[4];
     auto fetch = [&](int k0) {
         const int k = k0 + lch * 8;
         const bool kok = k < j.K;
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
+        for (int q = 0; q < 4; ++q) {
             ra[q] = (aok[q] && kok) ? *reinterpret_cast<const uint4 *>(ap[q] + k) : zero;
             rw[q] = (wok[q] && kok) ? *reinterpret_cast<const uint4 *>(wp[q] + k) : zero;
         }
     };
     fetch(0);
-    for (int k0 = 0; k0 < j.K; k0 += 32) {
+    for (int k0 = 0; k0 < j.K; k0 += KS) {
         if (j.src) {
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
+            for (int q = 0; q < 4; ++q) {
                 bf16_t *e = reinterpret_cast<bf16_t *>(&ra[q]);
 #pragma unroll
                 for (int y = 0; y < 8; ++y) st_f(e, y, ld_f(e, y) * rs[q]);
@@ -269,22 +271,25 @@ __device__ __forceinline__ void tile_product_mfma128(const TileJob &j, int row0,
         }
         __syncthreads();
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            *reinterpret_cast<uint4 *>(As + (lrow + 64 * q) * LD + lch * 8) = ra[q];
-            *reinterpret_cast<uint4 *>(Ws + (lrow + 64 * q) * LD + lch * 8) = rw[q];
+        for (int q = 0; q < 4; ++q) {
+            *reinterpret_cast<uint4 *>(As + (lrow + 32 * q) * LD + lch * 8) = ra[q];
+            *reinterpret_cast<uint4 *>(Ws + (lrow + 32 * q) * LD + lch * 8) = rw[q];
         }
         __syncthreads();
-        if (k0 + 32 < j.K) fetch(k0 + 32);
-        bf16x8 af[4], wf[4];
+        if (k0 + KS < j.K) fetch(k0 + KS);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            af[i] = *reinterpret_cast<const bf16x8 *>(As + (wr * 64 + i * 16 + lm) * LD + lq * 8);
-            wf[i] = *reinterpret_cast<const bf16x8 *>(Ws + (wc * 64 + i * 16 + lm) * LD + lq * 8);
+        for (int kk = 0; kk < KS; kk += 32) {
+            bf16x8 af[4], wf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                af[i] = *reinterpret_cast<const bf16x8 *>(As + (wr * 64 + i * 16 + lm) * LD + kk + lq * 8);
+                wf[i] = *reinterpret_cast<const bf16x8 *>(Ws + (wc * 64 + i * 16 + lm) * LD + kk + lq * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[c], acc[i][c], 0, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) acc[i][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[c], acc[i][c], 0, 0, 0);
     }
     bf16_t *y = (bf16_t *)j.y;
 #pragma unroll
@@ -303,7 +308,7 @@ __device__ __forceinline__ void tile_product_mfma128(const TileJob &j, int row0,
 }
 
 __global__ __launch_bounds__(256) void head_linear_mfma128_kernel(HeadLinearArgs p) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 40], Ws[128 * 40];
+    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 72], Ws[128 * 72];
     const int h = blockIdx.z;
     TileJob j{};
     j.a = (const bf16_t *)p.a + (int64_t)h * p.ha; j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)h * p.N * p.K; j.ldw = p.K;
@@ -313,7 +318,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma128_kernel(HeadLinearArgs
 }
 
 __global__ __launch_bounds__(256) void grouped_linear_mfma128_kernel(GroupedLinearArgs p) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 40], Ws[128 * 40];
+    __shared__ __attribute__((aligned(16))) bf16_t As[128 * 72], Ws[128 * 72];
     int tile = blockIdx.y, e = 0, lo = 0, hi = 0;
     for (; e < p.groups; ++e) {
         lo = p.off[e]; hi = p.off[e + 1];
@@ -528,6 +533,15 @@ __global__ __launch_bounds__(256) void side_gate_kernel(const OT *__restrict__ z
     st_f(g, idx, gelu_tanh_f(ld_f(z, idx)) * ld_f(E, ids[t] * lde + ecol + d));
 }
 
+// y[t][c] *= sigmoid(g[t][c])
+template <class OT>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(OT *__restrict__ y, int64_t ldy, const OT *__restrict__ g, int64_t ldg, int64_t T, int64_t N) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= T * N) return;
+    const int64_t t = idx / N, c = idx - t * N;
+    st_f(y, t * ldy + c, ld_f(y, t * ldy + c) * sigmoid_f(ld_f(g, t * ldg + c)));
+}
+
 template <class ET>
 __global__ __launch_bounds__(256) void embed_keep_kernel(const ET *__restrict__ E, const int64_t *__restrict__ ids, int W, float *__restrict__ x, float *__restrict__ kept) {
     const int64_t t = blockIdx.x, id = ids[t];
@@ -570,12 +584,12 @@ int group_norm(const GroupNormArgs &a, bool bf16, hipStream_t s) {
     return launched("group_norm");
 }
 
-int latent_store(const void *proj, int64_t ld, int64_t col, const Batch &b, int64_t rank, int64_t rot, float eps, const float *w, const float *freq, void *pages, bool bf16,
-                 hipStream_t s) {
+int latent_store(const void *proj, int64_t ld, int64_t col, const Batch &b, int64_t rank, int64_t rot, float eps, const float *w, const float *freq, void *pages, void *rows,
+                 bool bf16, hipStream_t s) {
     if (b.T == 0) return 0;
     if (rot % 2) return nvr::fail(NVR_ERR_INVALID_ARG, "latent_store: %ld rotated coordinates", (long)rot);
-    if (bf16) latent_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(64), 0, s>>>((const bf16_t *)proj, ld, col, b, (int)rank, (int)rot, eps, w, freq, (bf16_t *)pages);
-    else latent_store_kernel<float><<<dim3((unsigned)b.T), dim3(64), 0, s>>>((const float *)proj, ld, col, b, (int)rank, (int)rot, eps, w, freq, (float *)pages);
+    if (bf16) latent_store_kernel<bf16_t><<<dim3((unsigned)b.T), dim3(64), 0, s>>>((const bf16_t *)proj, ld, col, b, (int)rank, (int)rot, eps, w, freq, (bf16_t *)pages, (bf16_t *)rows);
+    else latent_store_kernel<float><<<dim3((unsigned)b.T), dim3(64), 0, s>>>((const float *)proj, ld, col, b, (int)rank, (int)rot, eps, w, freq, (float *)pages, (float *)rows);
     return launched("latent_store");
 }
 
@@ -650,6 +664,14 @@ int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, 
     if (bf16) moe_combine_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), 0, s>>>((const bf16_t *)y, place_of, (int)top, (const bf16_t *)shared, (int)W, (bf16_t *)out);
     else moe_combine_kernel<float><<<dim3((unsigned)T), dim3(256), 0, s>>>((const float *)y, place_of, (int)top, (const float *)shared, (int)W, (float *)out);
     return launched("moe_combine");
+}
+
+int sigmoid_gate(void *y, int64_t ldy, const void *g, int64_t ldg, int64_t T, int64_t N, bool bf16, hipStream_t s) {
+    if (T * N == 0) return 0;
+    const dim3 grid((unsigned)((T * N + 255) / 256));
+    if (bf16) sigmoid_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>((bf16_t *)y, ldy, (const bf16_t *)g, ldg, T, N);
+    else sigmoid_gate_kernel<float><<<grid, dim3(256), 0, s>>>((float *)y, ldy, (const float *)g, ldg, T, N);
+    return launched("sigmoid_gate");
 }
 
 int side_gate(const void *z, const int64_t *ids, const void *E, int64_t lde, int64_t ecol, int64_t dim, int64_t T, void *g, bool bf16, hipStream_t s) {

@@ -313,7 +313,7 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
         int64_t row = 0;
         for (size_t i = 0; i < nseq; ++i) {
             for (int64_t r0 = 0; r0 < (int64_t)seqs[i]->chunk_len; r0 += pw)
-                *tl++ = nvr::kt::FlashTile{(int32_t)(row + r0), (int32_t)std::min<int64_t>(pw, (int64_t)seqs[i]->chunk_len - r0), (int32_t)((int64_t)seqs[i]->chunk_start + r0), (int32_t)i};
+                *tl++ = nvr::kt::FlashTile{(int32_t)(row + r0), (int32_t)std::min<int64_t>(pw, (int64_t)seqs[i]->chunk_len - r0), (int32_t)((int64_t)seqs[i]->chunk_start + r0), flash_contiguous ? (int32_t)row : (int32_t)i};
             row += (int64_t)seqs[i]->chunk_len;
         }
     }
@@ -352,6 +352,8 @@ int LayeredModel::execute(nvr_model_runner &r, nvr_seq *const *seqs, size_t nseq
     bool decode_sized = true;
     for (size_t i = 0; i < nseq && decode_sized; ++i) decode_sized = seqs[i]->chunk_len == 1;
     StepPlan plan{b, d_want, (int64_t)R, T, max_ctx, o_tiles, n_tiles, o_ftiles, n_ftiles, decode_sized};
+    plan.whole_prompts = !decode_sized;
+    for (size_t i = 0; i < nseq && plan.whole_prompts; ++i) plan.whole_prompts = seqs[i]->chunk_start == 0;
     if (decode_sized && !r.cfg.enforce_eager) {
         const int64_t bucket = (max_ctx + 255) / 256 * 256;
         plan.max_ctx = plan.b.max_ctx = (int32_t)bucket;
@@ -466,6 +468,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
         return (int)NVR_OK;
     };
     lw.resize(spec.layers.size());
+    int64_t max_kvx = 0;
     int64_t max_nmix = 0, max_q2 = 0, max_qabs = 0, max_ctx = 0, max_hv = 0, max_qlat = 0, max_hd = 0, max_ff = 0, max_rows_e = 0, max_e2f = 0, max_ef = 0;
     size_t block_bytes = 0;
     for (size_t i = 0; i < spec.layers.size(); ++i) {
@@ -485,6 +488,19 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
             for (int64_t j = 0; j < R / 2; ++j) f[(size_t)j] = (float)std::pow(L.rot_base, -2.0 * (double)j / (double)L.rot_dims);
             RC(own(&w.rfreq, f.size() * 4)); NVR_HIP_CHECK(hipMemcpy(w.rfreq, f.data(), f.size() * 4, hipMemcpyHostToDevice));
             max_qabs = std::max(max_qabs, L.heads * (L.kv_rank + R)); max_ctx = std::max(max_ctx, L.heads * L.kv_rank);
+            // whole prompts (every key is a row of the step): keys and values expanded by one product and the dense graph's flash kernel, one key/value head per query head
+            w.flash = bf16 && L.dim + R == L.vdim && nvr::kb::flash_prefill_ok((int)L.vdim, (int)L.heads, (int)L.heads) && (L.kv_rank + R) % 32 == 0 && (2 * hv) % 16 == 0 &&
+                      w.nmix % 8 == 0 && (L.heads * (L.dim + R)) % 8 == 0;
+            if (w.flash) {
+                RC(own(&w.wx, (size_t)(2 * hv * (L.kv_rank + R) * esz)));
+                std::vector<uint16_t> one((size_t)1, f_to_bf16(1.0f));
+                for (int64_t h = 0; h < L.heads; ++h)           // the shared rotated key part is copied into every head's keys by rows of the identity
+                    for (int64_t j = 0; j < R; ++j)
+                        NVR_HIP_CHECK(hipMemcpy((char *)w.wx + (size_t)(((h * L.vdim + L.dim + j) * (L.kv_rank + R) + L.kv_rank + j) * esz), one.data(), 2, hipMemcpyHostToDevice));
+                if (std::find(flash_groups.begin(), flash_groups.end(), (int64_t)1) == flash_groups.end()) flash_groups.push_back(1);
+                flash_contiguous = true;
+                max_kvx = std::max(max_kvx, 2 * hv);
+            }
             // the matrix-core attention takes up to 16 query heads per key/value row: the heads go in equal shares of the largest divisor of H up to 16
             int64_t g = std::min<int64_t>(L.heads, 16);
             while (L.heads % g) --g;
@@ -528,12 +544,15 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
     rs.resize(spec.layers.size());
     for (size_t i = 0; i < spec.layers.size(); ++i) {
         const LayeredSpec::Layer &L = spec.layers[i];
-        if (L.mixer == LayeredSpec::LATENT && L.kv_from < 0) RC(named(&rs[i].kc, (size_t)(r.num_blocks * r.block_size * (L.kv_rank + L.rot_dim) * esz)));
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from < 0) {
+            RC(named(&rs[i].kc, (size_t)(r.num_blocks * r.block_size * (L.kv_rank + L.rot_dim) * esz)));
+            RC(own(&rs[i].rows, (size_t)(MT * (L.kv_rank + L.rot_dim) * esz)));                 // the step's own cached rows, in step order
+        }
         else if (L.mixer == LayeredSpec::GLA) RC(named((void **)&rs[i].state, (size_t)(slots * L.heads * L.dim * L.vdim * 4)));
     }
     for (size_t i = 0; i < spec.layers.size(); ++i) {                           // a layer without a latent of its own reads its source's pages
         const LayeredSpec::Layer &L = spec.layers[i];
-        if (L.mixer == LayeredSpec::LATENT && L.kv_from >= 0) { rs[i].kc = rs[(size_t)L.kv_from].kc; rs[i].borrowed = true; }
+        if (L.mixer == LayeredSpec::LATENT && L.kv_from >= 0) { rs[i].kc = rs[(size_t)L.kv_from].kc; rs[i].rows = rs[(size_t)L.kv_from].rows; rs[i].borrowed = true; }
     }
 
     // activations
@@ -544,6 +563,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
     RC(named((void **)&ret_o, (size_t)(MT * max_hv * 4))); RC(own(&az, (size_t)(MT * max_hd * esz)));
     RC(named(&gu, (size_t)(MT * max_ff * esz))); RC(own(&act, (size_t)(MT * max_ff * esz))); RC(own(&shared_y, (size_t)(MT * W * esz)));
     RC(own(&e_gu, (size_t)(MT * max_e2f * esz))); RC(own(&e_act, (size_t)(MT * max_ef * esz))); RC(own(&e_y, (size_t)(MT * max_rows_e * W * esz)));
+    RC(own(&kvx, (size_t)(MT * max_kvx * esz)));
     RC(own(&side_z, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz))); RC(own(&side_g, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz)));
     RC(own(&moe_i, (size_t)((3 * MT * std::max<int64_t>(max_rows_e, 1) + 1024 + 8) * 4))); RC(own(&moe_score, (size_t)(MT * std::max<int64_t>(max_rows_e, 1) * 4)));
     return NVR_OK;
@@ -592,13 +612,20 @@ int LayeredModel::load_sequential(nvr_model_runner &r, const std::string &name, 
         if (rest == "mix.g" && L.out_gate) return mat(rows_at(w.mix, w.gcol, W), W, hv, W);
         if (rest == "mix.dkv" && L.kv_from < 0) return mat(rows_at(w.mix, w.dcol, W), W, L.kv_rank + R, W);
         if (rest == "mix.dkv.norm" && L.kv_from < 0) return vec(w.dkvn, L.kv_rank);
-        if (rest == "mix.uv") return mat(w.uv, L.kv_rank, hv, L.kv_rank);
+        if (rest == "mix.uv") {
+            if (w.flash && is2(hv, L.kv_rank)) RC(put(r, (char *)w.wx + (size_t)(hv * (L.kv_rank + R) * esz), L.kv_rank + R, hv, L.kv_rank, dtype, data, true));
+            return mat(w.uv, L.kv_rank, hv, L.kv_rank);
+        }
         if (rest == "mix.uk") {                             // [H D][kv_rank] -> per head its transpose [kv_rank][D]: the expansion folds into the queries
             if (!is2(hd, L.kv_rank)) return bad();
             std::vector<float> t((size_t)(hd * L.kv_rank));
             for (int64_t h = 0; h < L.heads; ++h)
                 for (int64_t k = 0; k < L.dim; ++k)
                     for (int64_t n = 0; n < L.kv_rank; ++n) t[(size_t)((h * L.kv_rank + n) * L.dim + k)] = src_at(dtype, data, (size_t)((h * L.dim + k) * L.kv_rank + n));
+            if (w.flash)                                    // head h's key rows sit at h * (D + R) of the expansion (the rotated part's rows follow them)
+                for (int64_t h = 0; h < L.heads; ++h)
+                    RC(put(r, (char *)w.wx + (size_t)(h * L.vdim * (L.kv_rank + R) * esz), L.kv_rank + R, L.dim, L.kv_rank, dtype,
+                           (const char *)data + (size_t)(h * L.dim * L.kv_rank) * (dtype == 2 ? 4 : 2), true));
             return put(r, w.ukt, L.dim, L.heads * L.kv_rank, L.dim, 2, t.data(), true);
         }
     } else {
@@ -671,7 +698,19 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
                 RC(gemm(r, qlat, L.q_rank, w.uq, T, L.q_rank, L.heads * (L.dim + Rr), q2));
                 qsrc = q2; ldq = L.heads * (L.dim + Rr); qstride = L.dim + Rr;
             }
-            if (L.kv_from < 0) RC(kl::latent_store(proj, w.nmix, w.dcol, b, rank, Rr, eps, w.dkvn, w.rfreq, st.kc, bf16, s));
+            if (L.kv_from < 0) RC(kl::latent_store(proj, w.nmix, w.dcol, b, rank, Rr, eps, w.dkvn, w.rfreq, st.kc, st.rows, bf16, s));
+            if (w.flash && p.whole_prompts) {
+                // every key is a row of this step: K (with the rotated part) and V of all heads by one product from the step's cached rows, then the flash kernel
+                RC(kl::rotate_heads(qsrc, ldq, qstride, L.dim, b, L.heads, Rr, w.rfreq, (void *)qsrc, ldq, qstride, L.dim, bf16, s));   // (in place: a thread reads a pair, then writes it)
+                RC(gemm(r, st.rows, Dq, w.wx, T, Dq, 2 * hv, kvx));
+                const size_t gi = (size_t)(std::find(flash_groups.begin(), flash_groups.end(), (int64_t)1) - flash_groups.begin());
+                nvr::kt::FlashArgs f{};
+                f.q = (const uint16_t *)qsrc; f.ldq = ldq; f.k = (const uint16_t *)kvx; f.v = (const uint16_t *)kvx + hv; f.ldkv = 2 * hv;
+                f.tiles = (const nvr::kt::FlashTile *)(in_dev + p.o_ftiles[gi]); f.ntiles = p.n_ftiles[gi];
+                f.H = (int32_t)L.heads; f.KVH = (int32_t)L.heads; f.D = (int32_t)L.vdim; f.scale = (float)L.scale; f.out = (uint16_t *)cat; f.ldo = hv;
+                RC(nvr::kb::flash_prefill(f, false, s));
+                if (L.out_gate) RC(kl::sigmoid_gate(cat, hv, at(proj, w.gcol), w.nmix, T, hv, bf16, s));
+            } else {
             // the key expansion folded into the queries: per head q' = Wuk_h^T q (kv_rank numbers), then the rotated part
             kl::HeadLinearArgs ha{}; ha.a = qsrc; ha.lda = ldq; ha.ha = qstride; ha.w = w.ukt; ha.y = qabs; ha.ldy = L.heads * Dq; ha.hy = Dq;
             ha.T = (int32_t)T; ha.H = (int32_t)L.heads; ha.K = (int32_t)L.dim; ha.N = (int32_t)rank;
@@ -699,6 +738,7 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
             hu.T = (int32_t)T; hu.H = (int32_t)L.heads; hu.K = (int32_t)rank; hu.N = (int32_t)L.vdim;
             if (L.out_gate) { hu.gate = at(proj, w.gcol); hu.ldg = w.nmix; hu.hg = L.vdim; }
             RC(kl::head_linear(hu, bf16, s));
+            }
         } else {
             if (!w.wa1 || !w.wa2) return fail(NVR_ERR_NOT_ALLOCATED, "layer %ld: the decay projections were not loaded", (long)i);
             RC(gemm(r, a1, W, w.wa1, T, W, w.a_rank, alow));

@@ -72,6 +72,7 @@ public:
         int64_t qcol = 0, kcol = 0, vcol = 0, gcol = 0;
         // sequential layout
         float *n1 = nullptr, *n1b = nullptr, *n2 = nullptr, *n2b = nullptr;         // [W] each
+        void *wx = nullptr;                                 // latent attention: [2 H Dv][kv_rank + R], keys (with identity rows for the rotated part) then values of all heads
         int64_t head_share = 0;                             // latent attention on the matrix cores: query heads per launch
         int64_t dcol = 0;                                   // latent attention: column of the (queries' latent,) cached row's source in the mix projection
         void *uq = nullptr, *ukt = nullptr, *uv = nullptr, *wo = nullptr;            // [H (D + R)][q_rank]; [H][kv_rank][D] (Wuk per head, transposed); [H][Dv][kv_rank]; [W][H Dv]
@@ -81,7 +82,7 @@ public:
         float *router = nullptr; void *egu = nullptr, *edown = nullptr, *sgu = nullptr, *sdown = nullptr;   // [E][W] f32; [E][2 f][W]; [E][W][f]; [2 fs][W]; [W][fs]
         void *sgate = nullptr, *sproj = nullptr; float *snorm = nullptr, *dwa = nullptr;   // [side][W], [W][side], [W]; [i + 2]
     };
-    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; };   // borrowed: another run's pages (a shared latent)
+    struct RunState { void *kc = nullptr, *vc = nullptr; float *state = nullptr, *hist = nullptr; bool borrowed = false; void *rows = nullptr; };   // borrowed: another run's pages (a shared latent)
     std::vector<LayerW> lw;
     std::vector<RunState> rs;
     void *embed = nullptr, *head = nullptr; float gfinal = 1.f;
@@ -89,6 +90,7 @@ public:
     float *wfinal = nullptr; void *side_embed = nullptr;                    // [W]; [vocab][layers * side_dim]
     float *kept = nullptr;                                                  // the embedding output and every layer's output: [layers + 1][max tokens][W] f32
     void *qlat = nullptr, *q2 = nullptr, *qabs = nullptr, *ctx = nullptr, *alow = nullptr, *az = nullptr, *act = nullptr, *shared_y = nullptr;
+    bool flash_contiguous = false; void *kvx = nullptr;                      // flash tiles refer to rows of the step (not to block tables); expanded keys | values of a step
     int64_t alow_cap = 0; void *side_z = nullptr, *side_g = nullptr;
     void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
@@ -115,7 +117,7 @@ public:
 
 private:
     struct StepPlan { kl::Batch b; const int32_t *d_want; int64_t R, T, max_ctx; std::vector<size_t> o_tiles; std::vector<int32_t> n_tiles;
-                      std::vector<size_t> o_ftiles; std::vector<int32_t> n_ftiles; bool decode_sized; };
+                      std::vector<size_t> o_ftiles; std::vector<int32_t> n_ftiles; bool decode_sized; bool whole_prompts = false; };
     int forward(nvr_model_runner &r, const StepPlan &p);
     int init_sequential(nvr_model_runner &r);
     int load_sequential(nvr_model_runner &r, const std::string &name, int dtype, const int64_t *shape, int ndim, const void *data);
