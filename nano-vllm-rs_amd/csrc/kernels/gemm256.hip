@@ -44,6 +44,7 @@ struct G256Epi {
     int32_t H, KVH, D;
     int32_t kv_cache_only;             // GEPI_ROPE: k and v rows go to the caches only (the attention that follows reads them there)
     float *logits; float *pval; int32_t *pidx;   // GEPI_LMHEAD: f32 logits [T][N] (nullable), arg-max partials [tiles_x][T]
+    const int32_t *row_w; int64_t w_stride;      // GRP (rows grouped by expert): row block rb of 256 rows multiplies the matrix W + row_w[rb] * w_stride
 };
 
 constexpr int G_BK = 64, G_HT = 128, G_HALF = G_HT * G_BK * 2;          // 16 KiB per half-tile
@@ -67,7 +68,7 @@ __device__ __forceinline__ int g_w_uni(int hA, int i, int N) {
 
 // RD: head_dim of the RoPE variant as a compile-time constant (64 or 128; 0 for the other epilogues): its row map and pair geometry
 // fold to shifts, and the scalar registers they needed in the K loop are what pushed that variant into SGPR -> VGPR spills
-template <int EPI, int RD = 0>
+template <int EPI, int RD = 0, bool GRP = false>
 __global__ __launch_bounds__(512) void gemm256_kernel(const half_t *__restrict__ x, int64_t ldx, const half_t *__restrict__ W,
                                                       int T, int K, int N, int NW, half_t *__restrict__ y, G256Epi epi,
                                                       int tiles_x, int tiles_y, int CG) {
@@ -118,6 +119,7 @@ __global__ __launch_bounds__(512) void gemm256_kernel(const half_t *__restrict__
     auto set_sources = [&](int tile) {
         const int bx = tile % tiles_x, m0 = (tile / tiles_x) * 256;
         wb = W + (int64_t)bx * ((EPI == GEPI_SILU) ? 128 : 256) * K;
+        if (GRP) wb += (int64_t)epi.row_w[tile / tiles_x] * epi.w_stride;
         xb = x + (int64_t)m0 * ldx;
         rows_left = m0 + 256 > T ? T - 1 - m0 : 0x3fffffff;
         if (EPI == GEPI_LMHEAD) wrows_left = bx * 256 + 256 > N ? N - 1 - bx * 256 : 0x3fffffff;
@@ -493,7 +495,8 @@ static int g256_prepare() {                                               // 128
     if (done) return 0;
     const void *fns[] = {reinterpret_cast<const void *>(&gemm256_kernel<GEPI_F16>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_SILU>),
                          reinterpret_cast<const void *>(&gemm256_kernel<GEPI_ROPE, 128>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_ROPE, 64>),
-                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_RESID>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_LMHEAD>)};
+                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_RESID>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_LMHEAD>),
+                         reinterpret_cast<const void *>(&gemm256_kernel<GEPI_F16, 0, true>), reinterpret_cast<const void *>(&gemm256_kernel<GEPI_SILU, 0, true>)};
     for (const void *f : fns) {
         hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * G_BUF + 4096);
         if (e != hipSuccess) return nvr::fail(NVR_ERR_HIP, "gemm256: hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -534,6 +537,26 @@ int gemm256(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int6
     gemm256_kernel<GEPI_F16><<<dim3((unsigned)g256_grid(tt)), dim3(512), 2 * G_BUF, s>>>((const half_t *)x, ldx, (const half_t *)W, (int)T, (int)K,
                                                                                         (int)N, (int)N, (half_t *)y, G256Epi{}, tx, tt / tx, g256_cg(tx, tt / tx, false));
     return g256_check("gemm256");
+}
+// Rows grouped by expert (a mixture of experts over many tokens): T is a multiple of 256 and row block rb multiplies the matrix W + row_w[rb] * w_stride
+// (row_w on the device: the host does not know how many rows an expert got).  y = x . W_e^T, or out = silu(gate) * up with W_e = [gate rows; up rows].
+int gemm256_grouped(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s) {
+    if (!gemm256_ok(T, K, N, ldx) || T % 256) return nvr::fail(NVR_ERR_UNSUPPORTED, "gemm256_grouped: T=%ld K=%ld N=%ld", (long)T, (long)K, (long)N);
+    if (int rc = g256_prepare()) return rc;
+    G256Epi e{}; e.row_w = row_w; e.w_stride = w_stride;
+    const int tx = (int)(N / 256), tt = tx * (int)(T / 256);
+    gemm256_kernel<GEPI_F16, 0, true><<<dim3((unsigned)g256_grid(tt)), dim3(512), 2 * G_BUF, s>>>((const half_t *)x, ldx, (const half_t *)W, (int)T, (int)K, (int)N, (int)N, (half_t *)y, e, tx,
+                                                                                                  tt / tx, 0);
+    return g256_check("gemm256_grouped");
+}
+int gemm256_grouped_silu_mul(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t I, half_bits *out, hipStream_t s) {
+    if (!gemm256_silu_ok(T, K, I, ldx) || T % 256) return nvr::fail(NVR_ERR_UNSUPPORTED, "gemm256_grouped_silu_mul: T=%ld K=%ld I=%ld", (long)T, (long)K, (long)I);
+    if (int rc = g256_prepare()) return rc;
+    G256Epi e{}; e.row_w = row_w; e.w_stride = w_stride;
+    const int tx = (int)(I / 128), tt = tx * (int)(T / 256);
+    gemm256_kernel<GEPI_SILU, 0, true><<<dim3((unsigned)g256_grid(tt)), dim3(512), 2 * G_BUF, s>>>((const half_t *)x, ldx, (const half_t *)W, (int)T, (int)K, (int)I, (int)(2 * I), (half_t *)out, e,
+                                                                                                   tx, tt / tx, 0);
+    return g256_check("gemm256_grouped_silu_mul");
 }
 // h[T,N] <- fp16(h + fp16(x·Wᵀ)): the row-parallel GEMM with the residual add of qwen3.rs:382,389 in its epilogue (prefill steps on one
 // rank: the following norm then reads ONE tensor instead of h and the projection)

@@ -109,6 +109,8 @@ bool gemm256_ok(int64_t T, int64_t K, int64_t N, int64_t ldx);
 bool gemm256_silu_ok(int64_t T, int64_t K, int64_t I, int64_t ldx);
 bool gemm256_rope_ok(int64_t T, int64_t K, int64_t H, int64_t KVH, int64_t D, int64_t ldx);
 int gemm256(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s);
+int gemm256_grouped(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t N, half_bits *y, hipStream_t s);
+int gemm256_grouped_silu_mul(const half_bits *x, int64_t ldx, const half_bits *W, int64_t w_stride, const int32_t *row_w, int64_t T, int64_t K, int64_t I, half_bits *out, hipStream_t s);
 int gemm256_resid(const half_bits *x, int64_t ldx, const half_bits *W, int64_t T, int64_t K, int64_t N, half_bits *h, hipStream_t s);
 // LM head over >= 192 rows on the 256x256 tiles (f32 logits on demand + one arg-max partial per 256-column tile; any N % 16 == 0)
 bool gemm256_lm_head_ok(int64_t T, int64_t K, int64_t N, int64_t ldx);

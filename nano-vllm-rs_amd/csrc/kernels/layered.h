@@ -136,9 +136,12 @@ int poly_norm(const void *z, int64_t ldz, int64_t T, int64_t F, float eps, const
 int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool bf16, hipStream_t s);
 
 // Router of a mixture of experts: logits wr h in f32 (wr: [E][W] f32), the top largest per token -> sel / score (= sigmoid of the logit) [T][top]; then the rows
-// grouped by expert: off [E + 1], order [T top] (place -> token * top + choice), place_of (its inverse).
+// grouped by expert: off [E + 1], order [T top] (place -> token * top + choice), place_of (its inverse).  With pad > 1 every expert's rows start at a multiple of pad
+// (places then run up to (T top / pad + E) pad) and row_w[block] names the expert of each of the nblocks blocks of pad rows: the form a tiled product over whole
+// row blocks wants, with the rows brought together by moe_gather (xs[place] = h[token] * score).
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, bool bf16, hipStream_t s);
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s);
+int moe_gather(const void *h, int64_t ldh, int64_t T, int64_t W, int64_t top, const int32_t *place_of, const float *score, void *xs, bool bf16, hipStream_t s);
 // out[t] = sum_k y[place_of[t * top + k]] + shared[t] (shared may be null)
 int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s);
 

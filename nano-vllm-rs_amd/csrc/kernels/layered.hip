@@ -863,8 +863,8 @@ int retention(const RetentionArgs &a, const Batch &b, bool bf16, hipStream_t s) 
         else if (bf16) retention_seq_kernel<R_, bf16_t, false><<<grid, dim3(256), 0, s>>>(a, b);     \
         else retention_seq_kernel<R_, float, false><<<grid, dim3(256), 0, s>>>(a, b);                \
     } while (0)
-    if (a.D <= 256) {
-        const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
+    const size_t lds = ((size_t)(gated ? 3 : 2) * 16 * a.D + 16 * 32 + 16 * 8 * 32) * 4;
+    if (a.D <= 256 && lds <= 64 * 1024) {                 // (beyond: the token-by-token form, whose LDS does not grow with the key size)
 #define NVR_RETB(R_)                                                                                 \
     do {                                                                                             \
         if (gated) { if (bf16) retention_block_kernel<R_, bf16_t, true><<<grid, dim3(256), lds, s>>>(a, b);   \

@@ -452,16 +452,36 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const OT *__restrict__ h
 
 // One workgroup: counts per expert, offsets, and a place for every (token, choice) among its expert's rows.  order[place] = token * top + choice;
 // place_of[token * top + choice] = place.  Which place inside its expert a row gets is left to the atomics: a row's result does not depend on it.
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restrict__ sel, int n, int E, int32_t *__restrict__ off, int32_t *__restrict__ order,
-                                                         int32_t *__restrict__ place_of) {
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restrict__ sel, int n, int E, int pad, int nblocks, int32_t *__restrict__ off,
+                                                         int32_t *__restrict__ order, int32_t *__restrict__ place_of, int32_t *__restrict__ row_w) {
     extern __shared__ int32_t cnt[];                    // [E + 1] counts, then running offsets
     for (int e = threadIdx.x; e <= E; e += 1024) cnt[e] = 0;
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += 1024) atomicAdd(&cnt[sel[i]], 1);
     __syncthreads();
-    if (threadIdx.x == 0) { int run = 0; for (int e = 0; e < E; ++e) { const int c = cnt[e]; cnt[e] = run; off[e] = run; run += c; } off[E] = run; }
+    if (threadIdx.x == 0) {                             // an expert's rows start at a multiple of pad; row_w names the expert of every block of pad rows
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            const int c = cnt[e], padded = (c + pad - 1) / pad * pad;
+            cnt[e] = run; off[e] = run;
+            if (row_w) for (int bk = run / pad; bk < (run + padded) / pad && bk < nblocks; ++bk) row_w[bk] = e;
+            run += padded;
+        }
+        off[E] = run;
+        if (row_w) for (int bk = run / pad; bk < nblocks; ++bk) row_w[bk] = 0;      // (blocks behind the last expert: any matrix, their rows are nobody's)
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += 1024) { const int place = atomicAdd(&cnt[sel[i]], 1); order[place] = i; place_of[i] = place; }
+}
+
+// xs[place_of[i]] = h[i / top] * score[i] (the expert's input, in the order of the grouped rows)
+template <class OT>
+__global__ __launch_bounds__(256) void moe_gather_kernel(const OT *__restrict__ h, int64_t ldh, int W, int top, const int32_t *__restrict__ place_of, const float *__restrict__ score,
+                                                         OT *__restrict__ xs) {
+    const int64_t i = blockIdx.x, t = i / top;
+    const float sc = score[i];
+    OT *dst = xs + (int64_t)place_of[i] * W;
+    for (int c = threadIdx.x; c < W; c += 256) st_f(dst, c, ld_f(h, t * ldh + c) * sc);
 }
 
 // out[t] = sum_k y[place_of[t * top + k]] (+ shared[t]) in the operand type
@@ -648,15 +668,23 @@ int silu_mul(const void *gu, int64_t T, int64_t F, void *out, int64_t ldo, bool 
 }
 
 int moe_route(const void *h, int64_t ldh, int64_t T, int64_t W, const float *wr, int64_t E, int64_t top, int32_t *sel, float *score, int32_t *off, int32_t *order,
-              int32_t *place_of, bool bf16, hipStream_t s) {
+              int32_t *place_of, int64_t pad, int32_t *row_w, int64_t nblocks, bool bf16, hipStream_t s) {
     if (T == 0) return 0;
     if (top < 1 || top > E) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: %ld of %ld experts", (long)top, (long)E);
     if ((size_t)(E + 1) * 4 > 60000) return nvr::fail(NVR_ERR_UNSUPPORTED, "moe_route: %ld experts", (long)E);
     if (bf16) moe_route_kernel<bf16_t><<<dim3((unsigned)T), dim3(256), (size_t)E * 4, s>>>((const bf16_t *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score);
     else moe_route_kernel<float><<<dim3((unsigned)T), dim3(256), (size_t)E * 4, s>>>((const float *)h, ldh, (int)W, wr, (int)E, (int)top, sel, score);
     if (int rc = launched("moe_route")) return rc;
-    moe_group_kernel<<<dim3(1), dim3(1024), (size_t)(E + 1) * 4, s>>>(sel, (int)(T * top), (int)E, off, order, place_of);
+    if (pad < 1) return nvr::fail(NVR_ERR_INVALID_ARG, "moe_route: rows padded to %ld", (long)pad);
+    moe_group_kernel<<<dim3(1), dim3(1024), (size_t)(E + 1) * 4, s>>>(sel, (int)(T * top), (int)E, (int)pad, (int)nblocks, off, order, place_of, row_w);
     return launched("moe_group");
+}
+
+int moe_gather(const void *h, int64_t ldh, int64_t T, int64_t W, int64_t top, const int32_t *place_of, const float *score, void *xs, bool bf16, hipStream_t s) {
+    if (T * top == 0) return 0;
+    if (bf16) moe_gather_kernel<bf16_t><<<dim3((unsigned)(T * top)), dim3(256), 0, s>>>((const bf16_t *)h, ldh, (int)W, (int)top, place_of, score, (bf16_t *)xs);
+    else moe_gather_kernel<float><<<dim3((unsigned)(T * top)), dim3(256), 0, s>>>((const float *)h, ldh, (int)W, (int)top, place_of, score, (float *)xs);
+    return launched("moe_gather");
 }
 
 int moe_combine(const void *y, const int32_t *place_of, int64_t T, int64_t top, const void *shared, int64_t W, void *out, bool bf16, hipStream_t s) {

@@ -468,7 +468,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
         return (int)NVR_OK;
     };
     lw.resize(spec.layers.size());
-    int64_t max_kvx = 0;
+    int64_t max_kvx = 0, max_experts = 0, max_f = 0;
     int64_t max_nmix = 0, max_q2 = 0, max_qabs = 0, max_ctx = 0, max_hv = 0, max_qlat = 0, max_hd = 0, max_ff = 0, max_rows_e = 0, max_e2f = 0, max_ef = 0;
     size_t block_bytes = 0;
     for (size_t i = 0; i < spec.layers.size(); ++i) {
@@ -520,7 +520,7 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
             RC(own(&w.router, (size_t)(L.experts * W * 4)));
             RC(own(&w.egu, (size_t)(L.experts * 2 * f * W * esz))); RC(own(&w.edown, (size_t)(L.experts * W * f * esz)));
             if (fs) { RC(own(&w.sgu, (size_t)(2 * fs * W * esz))); RC(own(&w.sdown, (size_t)(W * fs * esz))); }
-            max_ff = std::max(max_ff, 2 * fs); max_rows_e = std::max(max_rows_e, L.top); max_e2f = std::max(max_e2f, L.top * 2 * f); max_ef = std::max(max_ef, L.top * f);
+            max_ff = std::max(max_ff, 2 * fs); max_rows_e = std::max(max_rows_e, L.top); max_e2f = std::max(max_e2f, L.top * 2 * f); max_ef = std::max(max_ef, L.top * f); max_experts = std::max(max_experts, L.experts); max_f = std::max(max_f, f);
         } else if (L.has_mlp) return fail(NVR_ERR_UNSUPPORTED, "layer %zu: this feed-forward does not belong to the sequential layout", i);
         if (spec.side_dim) { RC(own(&w.sgate, (size_t)(spec.side_dim * W * esz))); RC(own(&w.sproj, (size_t)(W * spec.side_dim * esz))); RC(own(&w.snorm, (size_t)W * 4)); }
         RC(own(&w.dwa, (size_t)(i + 2) * 4));                   // (until loaded: the layer's own output passes)
@@ -562,10 +562,12 @@ int LayeredModel::init_sequential(nvr_model_runner &r) {
     RC(own(&qlat, (size_t)(MT * max_qlat * esz))); RC(own(&q2, (size_t)(MT * max_q2 * esz))); RC(own(&qabs, (size_t)(MT * max_qabs * esz))); RC(own(&ctx, (size_t)(MT * max_ctx * esz)));
     RC(named((void **)&ret_o, (size_t)(MT * max_hv * 4))); RC(own(&az, (size_t)(MT * max_hd * esz)));
     RC(named(&gu, (size_t)(MT * max_ff * esz))); RC(own(&act, (size_t)(MT * max_ff * esz))); RC(own(&shared_y, (size_t)(MT * W * esz)));
-    RC(own(&e_gu, (size_t)(MT * max_e2f * esz))); RC(own(&e_act, (size_t)(MT * max_ef * esz))); RC(own(&e_y, (size_t)(MT * max_rows_e * W * esz)));
+    const int64_t pad_rows = (max_experts + 1) * 256;       // (experts' rows padded to whole blocks of 256)
+    RC(own(&e_gu, (size_t)(MT * max_e2f * esz))); RC(own(&e_act, (size_t)((MT * max_ef + pad_rows * max_f) * esz))); RC(own(&e_y, (size_t)((MT * max_rows_e + pad_rows) * W * esz)));
+    RC(own(&e_x, (size_t)((MT * max_rows_e + pad_rows) * W * esz)));
     RC(own(&kvx, (size_t)(MT * max_kvx * esz)));
     RC(own(&side_z, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz))); RC(own(&side_g, (size_t)(MT * std::max<int64_t>(spec.side_dim, 1) * esz)));
-    RC(own(&moe_i, (size_t)((3 * MT * std::max<int64_t>(max_rows_e, 1) + 1024 + 8) * 4))); RC(own(&moe_score, (size_t)(MT * std::max<int64_t>(max_rows_e, 1) * 4)));
+    RC(own(&moe_i, (size_t)((3 * MT * std::max<int64_t>(max_rows_e, 1) + max_experts + 1 + MT * std::max<int64_t>(max_rows_e, 1) / 256 + max_experts + 1024 + 8) * 4))); RC(own(&moe_score, (size_t)(MT * std::max<int64_t>(max_rows_e, 1) * 4)));
     return NVR_OK;
 }
 
@@ -763,14 +765,23 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
             RC(gemm(r, act, L.ff, w.down, T, L.ff, W, tmp));
         } else if (L.ff_kind == LayeredSpec::FF_MOE) {
             const int64_t f = L.expert_ff, fs = L.shared_ff, n = T * L.top;
-            int32_t *sel = moe_i, *order = sel + MT * L.top, *place_of = order + MT * L.top, *off = place_of + MT * L.top;
-            RC(kl::moe_route(a2, W, T, W, w.router, L.experts, L.top, sel, moe_score, off, order, place_of, bf16, s));
-            kl::GroupedLinearArgs g{}; g.a = a2; g.lda = W; g.w = w.egu; g.y = e_gu; g.ldy = 2 * f; g.off = off; g.groups = (int32_t)L.experts; g.K = (int32_t)W; g.N = (int32_t)(2 * f);
-            g.max_rows = (int32_t)n; g.src = order; g.rscale = moe_score; g.src_div = (int32_t)L.top;
-            RC(kl::grouped_linear(g, bf16, s));
-            RC(kl::silu_mul(e_gu, n, f, e_act, f, bf16, s));
-            kl::GroupedLinearArgs d{}; d.a = e_act; d.lda = f; d.w = w.edown; d.y = e_y; d.ldy = W; d.off = off; d.groups = (int32_t)L.experts; d.K = (int32_t)f; d.N = (int32_t)W; d.max_rows = (int32_t)n;
-            RC(kl::grouped_linear(d, bf16, s));
+            int32_t *sel = moe_i, *order = sel + MT * L.top, *place_of = order + MT * L.top, *off = place_of + MT * L.top, *row_w = off + L.experts + 1;
+            // many rows: every expert's rows padded to whole blocks of 256, brought together once, and the dense graph's 256 x 256 product with a matrix per row block
+            const int64_t nblocks = n / 256 + L.experts;
+            const bool blocks = bf16 && n >= 2048 && nvr::kb::gemm256_silu_ok(nblocks * 256, W, f, W) && nvr::kb::gemm256_ok(nblocks * 256, f, W, f);
+            RC(kl::moe_route(a2, W, T, W, w.router, L.experts, L.top, sel, moe_score, off, order, place_of, blocks ? 256 : 1, blocks ? row_w : nullptr, nblocks, bf16, s));
+            if (blocks) {
+                RC(kl::moe_gather(a2, W, T, W, L.top, place_of, moe_score, e_x, bf16, s));
+                RC(nvr::kb::gemm256_grouped_silu_mul((const uint16_t *)e_x, W, (const uint16_t *)w.egu, 2 * f * W, row_w, nblocks * 256, W, f, (uint16_t *)e_act, s));
+                RC(nvr::kb::gemm256_grouped((const uint16_t *)e_act, f, (const uint16_t *)w.edown, W * f, row_w, nblocks * 256, f, W, (uint16_t *)e_y, s));
+            } else {
+                kl::GroupedLinearArgs g{}; g.a = a2; g.lda = W; g.w = w.egu; g.y = e_gu; g.ldy = 2 * f; g.off = off; g.groups = (int32_t)L.experts; g.K = (int32_t)W; g.N = (int32_t)(2 * f);
+                g.max_rows = (int32_t)n; g.src = order; g.rscale = moe_score; g.src_div = (int32_t)L.top;
+                RC(kl::grouped_linear(g, bf16, s));
+                RC(kl::silu_mul(e_gu, n, f, e_act, f, bf16, s));
+                kl::GroupedLinearArgs d{}; d.a = e_act; d.lda = f; d.w = w.edown; d.y = e_y; d.ldy = W; d.off = off; d.groups = (int32_t)L.experts; d.K = (int32_t)f; d.N = (int32_t)W; d.max_rows = (int32_t)n;
+                RC(kl::grouped_linear(d, bf16, s));
+            }
             if (fs) {
                 RC(gemm(r, a2, W, w.sgu, T, W, 2 * fs, gu));
                 RC(kl::silu_mul(gu, T, fs, act, fs, bf16, s));

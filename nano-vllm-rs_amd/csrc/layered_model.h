@@ -92,6 +92,7 @@ public:
     void *qlat = nullptr, *q2 = nullptr, *qabs = nullptr, *ctx = nullptr, *alow = nullptr, *az = nullptr, *act = nullptr, *shared_y = nullptr;
     bool flash_contiguous = false; void *kvx = nullptr;                      // flash tiles refer to rows of the step (not to block tables); expanded keys | values of a step
     int64_t alow_cap = 0; void *side_z = nullptr, *side_g = nullptr;
+    void *e_x = nullptr;                                                    // experts' inputs gathered in the order of the grouped rows
     void *e_gu = nullptr, *e_act = nullptr, *e_y = nullptr; int32_t *moe_i = nullptr; float *moe_score = nullptr;
     std::vector<void *> owned;                                              // device allocations of the sequential layout (freed with the model)
     // activations

@@ -36,6 +36,7 @@ MECHANISMS = {
     "latent_attention_2_head_size_128_as_whole_prompt": make_config([latent2_layer(heads=2, dim=96, rot_dim=32, vdim=128, kv_rank=96, q_rank=64)], width=128, groups=4, side=0),
     "gla": make_config([gla_layer(heads=2, dim=24, vdim=32, tau=8.0)], side=0),
     "gla_tau_one_one_head": make_config([gla_layer(heads=1, dim=64, vdim=16, tau=1.0)], side=0),
+    "gla_keys_of_256": make_config([gla_layer(heads=1, dim=256, vdim=24, tau=4.0)], side=0),
     "gla_wide_keys": make_config([gla_layer(heads=1, dim=272, vdim=40, tau=16.0)], side=0),
     "dense_feed_forward": make_config([latent_layer(mlp=dense(80))], side=0),
     "experts_top_two_with_shared": make_config([latent_layer(mlp=moe(6, 2, 24, 40))], side=0),
@@ -70,6 +71,17 @@ def test_products_per_head_and_per_expert_with_many_rows(dtype):
     want = expected_logits(cfg, w, toks)
     check(Driver(cfg, w, dtype, page=16, pages=40, max_tokens=512).run_alone(toks), want, dtype, "one step")
     check(Driver(cfg, w, dtype, page=16, pages=40, max_tokens=512).run_alone(toks, cuts=[171, 129]), want, dtype, "two steps")
+
+
+def test_experts_over_whole_row_blocks():
+    """A step of more than two thousand expert rows at sizes the 256 x 256 product takes: the experts' rows are padded to whole blocks, gathered, and multiplied with
+    one matrix per block.  The same prompt in portions below that size takes the small tiles; both must agree with the restatement."""
+    cfg = make_config([latent_layer(heads=2, dim=32, vdim=32, kv_rank=64, mlp=moe(3, 2, 128, 128))], vocab=67, width=256, groups=4, side=0)
+    w = make_weights(cfg, seed=23)
+    toks = settled_tokens(cfg, w, 1100, 24)
+    want = expected_logits(cfg, w, toks)
+    check(Driver(cfg, w, "bfloat16", page=16, pages=80, max_tokens=1280, max_len=1280).run_alone(toks), want, "bfloat16", "one step")
+    check(Driver(cfg, w, "bfloat16", page=16, pages=80, max_tokens=1280, max_len=1280).run_alone(toks, cuts=[400]), want, "bfloat16", "portions of 400")
 
 
 def test_each_part_changes_the_result():
