@@ -335,6 +335,92 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma128_kernel(GroupedLine
     tile_product_mfma128(j, tile * 128, blockIdx.x * 128, As, Ws);
 }
 
+// Few rows (decode-sized steps, experts with a handful of tokens): a 16 x 64 tile per workgroup and the four waves split K, so that a product whose cost is
+// reading the matrix is spread over four times as many workgroups; the partial sums meet in LDS.
+__device__ __forceinline__ void tile_product_mfma_ksplit(const TileJob &j, int row0, int col0, float *part) {      // part: [3][16 * 64] floats of LDS
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4;
+    const bf16_t *w = (const bf16_t *)j.w;
+    const int r = row0 + lm;
+    const bool rok = r < j.rows;
+    const bf16_t *ap = (const bf16_t *)j.a; float rs = 1.f;
+    if (rok) {
+        if (j.src) { const int sidx = j.src[r]; ap += (int64_t)(sidx / j.src_div) * j.lda; rs = j.rscale[sidx]; }
+        else ap += (int64_t)r * j.lda;
+    }
+    const bf16_t *wp[4]; bool cok[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) { const int n = col0 + cb * 16 + lm; cok[cb] = n < j.N; wp[cb] = w + (int64_t)(cok[cb] ? n : 0) * j.ldw; }
+    f32x4 acc[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) acc[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const uint4 zero{0, 0, 0, 0};
+    const int kq = ((j.K + 3) / 4 + 31) / 32 * 32, kbeg = wave * kq, kend = min(j.K, kbeg + kq);
+#pragma unroll 2
+    for (int k0 = kbeg; k0 < kend; k0 += 32) {
+        const int k = k0 + lq * 8;
+        const bool kok = k < kend;
+        uint4 av = (rok && kok) ? *reinterpret_cast<const uint4 *>(ap + k) : zero;
+        uint4 wv[4];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) wv[cb] = (cok[cb] && kok) ? *reinterpret_cast<const uint4 *>(wp[cb] + k) : zero;
+        if (j.src) {
+            bf16_t *e = reinterpret_cast<bf16_t *>(&av);
+#pragma unroll
+            for (int y = 0; y < 8; ++y) st_f(e, y, ld_f(e, y) * rs);
+        }
+        const bf16x8 af = __builtin_bit_cast(bf16x8, av);
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, __builtin_bit_cast(bf16x8, wv[cb]), acc[cb], 0, 0, 0);
+    }
+    if (wave > 0)
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[(wave - 1) * 1024 + (lq * 4 + i) * 64 + cb * 16 + lm] = acc[cb][i];
+    __syncthreads();
+    if (wave > 0) return;
+    bf16_t *y = (bf16_t *)j.y;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int rr = row0 + lq * 4 + i, n = col0 + cb * 16 + lm, at = (lq * 4 + i) * 64 + cb * 16 + lm;
+            if (rr < j.rows && n < j.N) {
+                float v = (acc[cb][i] + part[at]) + (part[1024 + at] + part[2048 + at]);
+                if (j.gate) v *= sigmoid_f(ld_f((const bf16_t *)j.gate, (int64_t)rr * j.ldg + n));
+                st_f(y, (int64_t)rr * j.ldy + n, v);
+            }
+        }
+}
+
+__global__ __launch_bounds__(256) void head_linear_ksplit_kernel(HeadLinearArgs p) {
+    __shared__ float part[3 * 1024];
+    const int h = blockIdx.z;
+    TileJob j{};
+    j.a = (const bf16_t *)p.a + (int64_t)h * p.ha; j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)h * p.N * p.K; j.ldw = p.K;
+    j.y = (bf16_t *)p.y + (int64_t)h * p.hy; j.ldy = p.ldy; j.rows = p.T; j.K = p.K; j.N = p.N;
+    j.gate = p.gate ? (const void *)((const bf16_t *)p.gate + (int64_t)h * p.hg) : nullptr; j.ldg = p.ldg;
+    tile_product_mfma_ksplit(j, blockIdx.y * 16, blockIdx.x * 64, part);
+}
+
+__global__ __launch_bounds__(256) void grouped_linear_ksplit_kernel(GroupedLinearArgs p) {
+    __shared__ float part[3 * 1024];
+    int tile = blockIdx.y, e = 0, lo = 0, hi = 0;
+    for (; e < p.groups; ++e) {
+        lo = p.off[e]; hi = p.off[e + 1];
+        const int nt = (hi - lo + 15) >> 4;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (e == p.groups) return;                              // (the whole workgroup leaves)
+    TileJob j{};
+    j.lda = p.lda; j.w = (const bf16_t *)p.w + (int64_t)e * p.N * p.K; j.ldw = p.K; j.y = (bf16_t *)p.y + (int64_t)lo * p.ldy; j.ldy = p.ldy;
+    j.rows = hi - lo; j.K = p.K; j.N = p.N;
+    if (p.src) { j.a = p.a; j.src = p.src + lo; j.rscale = p.rscale; j.src_div = p.src_div; }
+    else j.a = (const bf16_t *)p.a + (int64_t)lo * p.lda;
+    tile_product_mfma_ksplit(j, tile * 16, blockIdx.x * 64, part);
+}
+
 template <int WR>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinearArgs p) {
     const int h = blockIdx.z;
@@ -628,7 +714,7 @@ int head_linear(const HeadLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.T == 0 || a.N == 0 || a.H == 0) return 0;
     if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && a.ha % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
         if (a.T >= 128) head_linear_mfma128_kernel<<<dim3((unsigned)((a.N + 127) / 128), (unsigned)((a.T + 127) / 128), (unsigned)a.H), dim3(256), 0, s>>>(a);
-        else if (a.T <= 16) head_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)((a.T + 15) / 16), (unsigned)a.H), dim3(256), 0, s>>>(a);
+        else if (a.T <= 16) head_linear_ksplit_kernel<<<dim3((unsigned)((a.N + 63) / 64), (unsigned)((a.T + 15) / 16), (unsigned)a.H), dim3(256), 0, s>>>(a);
         else head_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)((a.T + 63) / 64), (unsigned)a.H), dim3(256), 0, s>>>(a);
         return launched("head_linear");
     }
@@ -642,7 +728,7 @@ int grouped_linear(const GroupedLinearArgs &a, bool bf16, hipStream_t s) {
     if (a.max_rows == 0 || a.N == 0 || a.groups == 0) return 0;
     if (bf16 && a.K % 8 == 0 && a.lda % 8 == 0 && aligned16(a.a) && aligned16(a.w)) {
         if (a.max_rows >= 96 * a.groups) grouped_linear_mfma128_kernel<<<dim3((unsigned)((a.N + 127) / 128), (unsigned)(a.max_rows / 128 + a.groups)), dim3(256), 0, s>>>(a);
-        else if (a.max_rows <= 16 * a.groups) grouped_linear_mfma_kernel<1><<<dim3((unsigned)((a.N + 255) / 256), (unsigned)(a.max_rows / 16 + a.groups)), dim3(256), 0, s>>>(a);
+        else if (a.max_rows <= 16 * a.groups) grouped_linear_ksplit_kernel<<<dim3((unsigned)((a.N + 63) / 64), (unsigned)(a.max_rows / 16 + a.groups)), dim3(256), 0, s>>>(a);
         else grouped_linear_mfma_kernel<4><<<dim3((unsigned)((a.N + 63) / 64), (unsigned)(a.max_rows / 64 + a.groups)), dim3(256), 0, s>>>(a);
         return launched("grouped_linear");
     }
