@@ -530,6 +530,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const OT *__restrict__ h
                 const float ob = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
                 if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
             }
+            if (bi >= E) bi = E - 1;                        // (logits that are not numbers compare false everywhere: the index still has to be an expert's)
             if (lane == 0) { sel[t * top + k] = bi; score[t * top + k] = sigmoid_f(best); sc[bi] = -INFINITY; }
         }
         __syncthreads();

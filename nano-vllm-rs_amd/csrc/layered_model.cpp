@@ -783,8 +783,11 @@ int LayeredModel::forward_sequential(nvr_model_runner &r, const StepPlan &p) {
                 RC(kl::grouped_linear(d, bf16, s));
             }
             if (fs) {
-                RC(gemm(r, a2, W, w.sgu, T, W, 2 * fs, gu));
-                RC(kl::silu_mul(gu, T, fs, act, fs, bf16, s));
+                if (bf16 && nvr::kb::gemm256_silu_ok(T, W, fs, W)) RC(nvr::kb::gemm256_silu_mul((const uint16_t *)a2, W, (const uint16_t *)w.sgu, T, W, fs, (uint16_t *)act, s));   // (gate, up and SiLU in one launch)
+                else {
+                    RC(gemm(r, a2, W, w.sgu, T, W, 2 * fs, gu));
+                    RC(kl::silu_mul(gu, T, fs, act, fs, bf16, s));
+                }
                 RC(gemm(r, act, fs, w.sdown, T, fs, W, shared_y));
             }
             RC(kl::moe_combine(e_y, place_of, T, L.top, fs ? shared_y : nullptr, W, tmp, bf16, s));
